@@ -1,0 +1,61 @@
+"""Device side of the cache: page storage for every run that keeps keys and values, state
+rows for every run that keeps state, and the grouping of runs by need.
+
+Page tensors are ``[pages + 1, kv_heads, page_size, head_dim]`` in the engine's type, zeroed
+once (page 0, the null page, stays zero and is never written).  Layout and zero-init follow
+``jllm/engine/paged.py:26-38`` except that the head axis comes before the slot axis, so one
+head's keys of a page are contiguous for the attention kernels.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..parts.spec import LayerMemory
+
+_STATE_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32}
+
+
+def group_keys_of(plan) -> list:
+    """Distinct cache needs in schedule order of first appearance."""
+    keys = []
+    for p in plan:
+        if p.cache is not None and p.cache_of is None and p.cache.group_key not in keys:
+            keys.append(p.cache.group_key)
+    return keys
+
+
+def has_state(plan) -> bool:
+    return any(p.state is not None for p in plan)
+
+
+def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs: int, dtype, device) -> list:
+    """One ``LayerMemory`` per schedule entry.  ``num_pages``: usable pages per group."""
+    if isinstance(num_pages, int):
+        num_pages = [num_pages] * len(group_keys)
+    memories = []
+    for p in plan:
+        mem = LayerMemory()
+        if p.cache is not None:
+            if p.cache_of is None:
+                g = group_keys.index(p.cache.group_key)
+                shape = (num_pages[g] + 1, p.cache.num_kv_heads, page_size, p.cache.head_dim)
+                mem.k_pages = torch.zeros(shape, dtype=dtype, device=device)
+                mem.v_pages = torch.zeros(shape, dtype=dtype, device=device)
+                mem.group, mem.writes = g, True
+            else:
+                owner = memories[p.cache_of]
+                if owner.k_pages is None:
+                    raise ValueError(f"run {p.run} reads the cache of run {p.cache_of}, which keeps none")
+                own, other = p.cache, plan[p.cache_of].cache
+                if (own.num_kv_heads, own.head_dim) != (other.num_kv_heads, other.head_dim):
+                    raise ValueError(f"run {p.run} cannot read run {p.cache_of}'s cache: head shapes differ")
+                mem.k_pages, mem.v_pages, mem.group, mem.writes = owner.k_pages, owner.v_pages, owner.group, False
+        if p.state is not None:
+            mem.state = torch.zeros((max_num_seqs, *p.state.shape), dtype=_STATE_DTYPES[p.state.dtype], device=device)
+        memories.append(mem)
+    return memories
+
+
+def cache_bytes_per_token(plan, dtype) -> int:
+    item = torch.empty((), dtype=dtype).element_size()
+    return sum(2 * p.cache.num_kv_heads * p.cache.head_dim * item for p in plan if p.cache and p.cache_of is None)

@@ -1,0 +1,162 @@
+"""The step function and what it stands on: a bound model, the cache manager, the device
+memory of every layer.
+
+One call of ``EngineCore.run`` takes a batch of (request, its next tokens): portions of
+prompts beside single decoded tokens, cut anywhere.  It runs only those tokens, as one
+flattened batch, against what earlier steps left in the cache, stores their keys and
+values, and returns float logits at the places asked for.  The reference has two device
+programs instead, a prefill of exactly one block per row and a decode of one token per
+row, padded to bucket shapes (``jllm/engine/generate.py:112-143, 233-265``,
+``jllm/engine/engine.py:317-496``); their per-row arguments (``pos_starts``, block tables,
+``valid_tokens``, ``last_token_idx``, ``phys_blocks``, ``slot_in_block``) are what the
+flattened arrays built here carry per token and per request.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.storage import allocate_memories, cache_bytes_per_token, group_keys_of, has_state
+from ..config.engine import EngineConfig
+from ..parts.model import DecoderModel
+from ..parts.spec import StepContext
+from ..weights.loader import TORCH_DTYPES
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens and the indices among them (0-based)
+    whose logits are wanted."""
+
+    request_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)
+
+
+class EngineCore:
+    def __init__(self, model: DecoderModel, config: EngineConfig, num_pages=None):
+        """``num_pages`` overrides the configuration's usable pages per cache group."""
+        if model.dtype != TORCH_DTYPES[config.dtype]:
+            raise ValueError(f"model is bound in {model.dtype}, the engine is configured for {config.dtype}")
+        self.model, self.config = model, config
+        self.device = model.device
+        self.dtype = model.dtype
+        self.page_size = config.page_size
+        self.plan = model.memory_plan()
+        self.group_keys = group_keys_of(self.plan)
+        pages = num_pages if num_pages is not None else config.usable_pages
+        self.cache = CacheManager(self.group_keys, self.page_size, pages, config.max_num_seqs,
+                                  config.enable_prefix_cache, has_state(self.plan))
+        self.memories = allocate_memories(self.plan, self.group_keys, pages, self.page_size,
+                                          config.max_num_seqs, self.dtype, self.device)
+        self.vocab_size = model.spec.vocab_size
+        self.kv_bytes_per_token = cache_bytes_per_token(self.plan, self.dtype)
+
+    # ---- requests
+    def start_request(self, request_id, prompt: Optional[Sequence[int]] = None) -> int:
+        """Returns the number of prompt tokens found in the prefix cache (0 without a prompt)."""
+        return self.cache.start(request_id, prompt)
+
+    def finish_request(self, request_id) -> None:
+        self.cache.finish(request_id)
+
+    def has_request(self, request_id) -> bool:
+        return self.cache.has(request_id)
+
+    # ---- the step
+    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Float logits [wanted, vocab] in the order of the entries and of their ``want``.
+        Raises ``OutOfPages`` before anything ran if a request's tokens have no room."""
+        entries = [e for e in entries if len(e.tokens) > 0]
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
+        for e in entries:
+            for t in e.tokens:
+                if not 0 <= int(t) < self.vocab_size:
+                    raise ValueError(f"request {e.request_id!r}: token id {t} outside the vocabulary [0, {self.vocab_size})")
+            for w in e.want:
+                if not 0 <= int(w) < len(e.tokens):
+                    raise ValueError(f"request {e.request_id!r}: wanted place {w} outside its {len(e.tokens)} tokens")
+        for e in entries:
+            self.cache.reserve(e.request_id, len(e.tokens))
+        token_ids, ctx, logit_rows = self._build(entries)
+        self._zero_new_state()
+        logits = self.model.forward(token_ids, ctx, self.memories, logit_rows)
+        for e in entries:
+            self.cache.commit(e.request_id, e.tokens)
+        return logits
+
+    def _zero_new_state(self) -> None:
+        slots = self.cache.take_new_slots()
+        if slots and any(m.state is not None for m in self.memories):
+            idx = torch.tensor(slots, dtype=torch.long, device=self.device)
+            for m in self.memories:
+                if m.state is not None:
+                    m.state.index_fill_(0, idx, 0)
+
+    def _build(self, entries):
+        """All per-token and per-request integers of the step, packed on the host into one
+        pinned buffer and copied to the device at once."""
+        cache, ps = self.cache, self.page_size
+        n_groups = len(self.group_keys)
+        q_lens = [len(e.tokens) for e in entries]
+        ctx_lens = [cache.context_len(e.request_id) for e in entries]
+        slots = [cache.slot(e.request_id) for e in entries]
+        n, r = sum(q_lens), len(entries)
+        tables = [[cache.block_table(e.request_id, g) for e in entries] for g in range(n_groups)]
+        widths = [max(1, max(len(t) for t in tables[g])) for g in range(n_groups)]
+        m = sum(len(e.want) for e in entries)
+
+        sizes = [n, n, n, r + 1, r, r, m] + [n] * n_groups + [r * w for w in widths]
+        offsets = np.concatenate([[0], np.cumsum(sizes)])
+        buf = torch.empty(int(offsets[-1]), dtype=torch.int32, pin_memory=True)
+        host = buf.numpy()
+
+        def seg(i):
+            return host[offsets[i]:offsets[i + 1]]
+
+        tok, pos, treq, cu, ctxl, slot_ids, rows = (seg(i) for i in range(7))
+        cu[0] = 0
+        at, row_at = 0, 0
+        for i, e in enumerate(entries):
+            ql = q_lens[i]
+            tok[at:at + ql] = np.asarray(e.tokens, dtype=np.int32)
+            pos[at:at + ql] = np.arange(ctx_lens[i], ctx_lens[i] + ql, dtype=np.int32)
+            treq[at:at + ql] = i
+            for w in e.want:
+                rows[row_at] = at + int(w)
+                row_at += 1
+            at += ql
+            cu[i + 1] = at
+        ctxl[:] = ctx_lens
+        slot_ids[:] = slots
+        for g in range(n_groups):
+            sm = seg(7 + g)
+            at = 0
+            for i, e in enumerate(entries):
+                sm[at:at + q_lens[i]] = cache.slot_mapping(e.request_id, g, q_lens[i])
+                at += q_lens[i]
+            bt = seg(7 + n_groups + g).reshape(r, widths[g])
+            bt[:] = 0
+            for i, t in enumerate(tables[g]):
+                bt[i, :len(t)] = t
+
+        dev = buf.to(self.device, non_blocking=True)
+
+        def dseg(i):
+            return dev[int(offsets[i]):int(offsets[i + 1])]
+
+        ctx = StepContext(
+            num_tokens=n, num_requests=r, positions=dseg(1), token_req=dseg(2), cu_seqlens=dseg(3),
+            context_lens=dseg(4), slot_ids=dseg(5),
+            block_tables=[dseg(7 + n_groups + g).view(r, widths[g]) for g in range(n_groups)],
+            slot_mappings=[dseg(7 + g) for g in range(n_groups)],
+            page_size=ps, q_lens_host=q_lens, context_lens_host=ctx_lens, slot_ids_host=slots,
+            max_q_len=max(q_lens), max_kv_len=max(c + q for c, q in zip(ctx_lens, q_lens)),
+        )
+        ctx.extras["pinned"] = buf  # keeps the staging buffer alive until the step has run
+        return dseg(0), ctx, dseg(6)

@@ -1,0 +1,143 @@
+"""The Python entry point: an engine object with ``add_request / step / has_work`` and a
+blocking ``generate``, plus module-level functions in the reference's own manner
+(``make_driver``, ``add_request(driver, ...)``, ``step(driver)``, ``has_work(driver)``:
+``jllm/engine/engine.py:63-168``; the canonical loop is ``tests/_greedy.py:34-43``).
+Tokens in, tokens out: tokenisers are not part of the engine.
+"""
+from __future__ import annotations
+
+from pathlib import Path
+from typing import Mapping, Optional, Sequence, Union
+
+from ..config.engine import EngineConfig
+from ..sampling.sampler import Sampler, draw_key
+from .core import EngineCore, StepEntry
+from .request import EngineStats, Request, SamplingParams, StepEvent
+from .scheduler import Scheduler
+
+
+class LLM:
+    """One model on one GPU behind a continuous-batching scheduler.
+
+    ``model`` is a model folder (``config.json`` + safetensors), or a ``config.json``-style
+    dict for random weights drawn on the device from ``random_seed``, or an already bound
+    ``DecoderModel``.  The other arguments are the fields of ``EngineConfig``; the reference's
+    names (``max_num_seqs``, ``max_model_len``, ``max_prefill_len``, ``block_size``,
+    ``num_blocks``, ``dtype`` = "bf16" | "fp32") keep their meaning.
+    """
+
+    def __init__(self, model, *, random_seed: int = 0, device="cuda", **engine_options):
+        from ..parts.model import DecoderModel
+        from ..weights import load_model, random_model_on_device
+
+        self.config = EngineConfig(**engine_options)
+        if isinstance(model, DecoderModel):
+            self.model = model
+        elif isinstance(model, Mapping):
+            self.model, self.model_config = random_model_on_device(model, random_seed, self.config.dtype, device=device)
+        else:
+            self.model, self.model_config = load_model(Path(model), self.config.dtype, device)
+        self.core = EngineCore(self.model, self.config)
+        self.stats = EngineStats()
+        self.scheduler = Scheduler(self.config, self.core.cache, self.stats)
+        self.sampler = Sampler(self.core.device)
+        self._next_id = 0
+        self.requests: dict = {}
+
+    # ---- the reference's loop: add_request / has_work / step
+    def add_request(self, prompt_ids: Sequence[int], sampling: Optional[SamplingParams] = None,
+                    arrival_step: int = 0) -> int:
+        sp = sampling or SamplingParams()
+        vocab = self.core.vocab_size
+        for t in prompt_ids:
+            if not 0 <= int(t) < vocab:
+                raise ValueError(f"token id {t} outside the vocabulary [0, {vocab})")
+        if sp.max_new_tokens < 1:
+            raise ValueError("max_new_tokens must be at least 1")
+        rid = self._next_id
+        req = Request(request_id=rid, prompt_ids=[int(t) for t in prompt_ids], sampling=sp, arrival_step=arrival_step)
+        self.scheduler.add(req)
+        self._next_id += 1
+        self.requests[rid] = req
+        return rid
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    def step(self) -> list:
+        """One scheduler iteration: schedule, run the mixed batch, sample, finish.  Returns the
+        ``StepEvent`` of every token emitted."""
+        out = self.scheduler.schedule()
+        if not out.items:
+            return []
+        entries, sampled = [], []
+        for item in out.items:
+            req = item.request
+            tokens = req.all_tokens[req.num_computed:req.num_computed + item.num_tokens]
+            entries.append(StepEntry(req.request_id, tokens, [item.num_tokens - 1] if item.samples else []))
+            if item.samples:
+                sampled.append(item)
+            if item.num_tokens == 1 and item.samples and req.output_ids:
+                self.stats.decode_tokens += 1
+                self.stats.decode_calls += 1
+            else:
+                self.stats.prefill_tokens += item.num_tokens
+                self.stats.prefill_portions += 1
+        self.stats.steps_run += 1
+        self.stats.max_batched_tokens = max(self.stats.max_batched_tokens, out.num_tokens)
+        logits = self.core.run(entries)
+        temps = [i.request.sampling.temperature for i in sampled]
+        keys = [
+            draw_key(i.request.sampling.seed if i.request.sampling.seed is not None else self.config.seed,
+                     i.request.request_id, len(i.request.output_ids))
+            for i in sampled
+        ]
+        tokens = self.sampler.sample(logits, temps, keys)
+        events, k = [], 0
+        for item in out.items:
+            tok = None
+            if item.samples:
+                tok = tokens[k]
+                k += 1
+            finished = self.scheduler.advance(item, tok)
+            if tok is not None:
+                self.stats.emitted_tokens += 1
+                events.append(StepEvent(item.request.request_id, int(tok), finished))
+        return events
+
+    # ---- blocking use
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 sampling: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 arrival_steps: Optional[Sequence[int]] = None) -> list:
+        """Generated token ids of every prompt, in the order given."""
+        if sampling is None or isinstance(sampling, SamplingParams):
+            sampling = [sampling or SamplingParams()] * len(prompts)
+        arrival_steps = arrival_steps or [0] * len(prompts)
+        rids = [self.add_request(p, s, a) for p, s, a in zip(prompts, sampling, arrival_steps)]
+        while self.has_work():
+            self.step()
+        outs = [list(self.requests[r].output_ids) for r in rids]
+        for r in rids:
+            del self.requests[r]
+        return outs
+
+
+# ---- the reference's functional spelling ------------------------------------------------
+def make_driver(model, max_num_seqs: int, max_model_len: int, max_prefill_len: Optional[int] = None,
+                block_size: int = 16, num_blocks: Optional[int] = None, dtype: str = "bf16", **more) -> LLM:
+    """``jllm/engine/engine.py:63-109`` with the same argument names.  ``model``: folder, config
+    dict or bound model.  ``num_blocks`` below the worst case is allowed here."""
+    return LLM(model, max_num_seqs=max_num_seqs, max_model_len=max_model_len, max_prefill_len=max_prefill_len,
+               block_size=block_size, num_blocks=num_blocks, dtype=dtype, **more)
+
+
+def add_request(driver: LLM, prompt_ids, sampling: Optional[SamplingParams] = None) -> int:
+    return driver.add_request(prompt_ids, sampling)
+
+
+def has_work(driver: LLM) -> bool:
+    return driver.has_work()
+
+
+def step(driver: LLM) -> list:
+    return driver.step()

@@ -1,0 +1,262 @@
+"""Typed Python entry points of the HIP kernels.
+
+Every wrapper checks on the host that the operands have the device, type,
+contiguity and shapes that the kernel and its grid assume, then launches on
+torch's current stream.  There is no other implementation behind these
+functions: a missing library raises ``KernelLibraryError``.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_void_p
+
+import torch
+
+from . import library
+
+_SUFFIX = {torch.bfloat16: "bf16", torch.float32: "f32"}
+
+
+class KernelArgumentError(ValueError):
+    """An operand does not have the shape, type or layout the kernel needs."""
+
+
+def _suffix(dtype: torch.dtype) -> str:
+    try:
+        return _SUFFIX[dtype]
+    except KeyError:
+        raise KernelArgumentError(f"kernels take bfloat16 or float32, not {dtype}") from None
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t) -> c_void_p:
+    return c_void_p(0 if t is None else t.data_ptr())
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise KernelArgumentError(msg)
+
+
+def _dev(*tensors) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel operands must live on the GPU")
+            _need(t.is_contiguous(), "kernel operands must be contiguous")
+
+
+def _check(code: int, name: str) -> None:
+    if code != 0:
+        raise RuntimeError(f"{name}: HIP error {code}")
+
+
+def _i32(t, name: str, n: int | None = None) -> None:
+    _need(t.dtype == torch.int32, f"{name} must be int32")
+    if n is not None:
+        _need(t.numel() == n, f"{name} must have {n} entries, has {t.numel()}")
+
+
+def _f32(t, name: str, n: int | None = None) -> None:
+    _need(t.dtype == torch.float32, f"{name} must be float32")
+    if n is not None:
+        _need(t.numel() == n, f"{name} must have {n} entries, has {t.numel()}")
+
+
+# --------------------------------------------------------------------------- embedding
+def embedding(h: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    """h[t] = float(table[ids[t]]); ids must already be checked to lie in [0, rows)."""
+    _dev(h, table, ids)
+    n, hidden = h.shape
+    _f32(h, "h")
+    _i32(ids, "ids", n)
+    _need(table.dim() == 2 and table.shape[1] == hidden, "table width differs from h")
+    fn = getattr(library.core(), f"jv_embedding_{_suffix(table.dtype)}")
+    _check(fn(_ptr(h), _ptr(table), _ptr(ids), c_int(n), c_int(hidden), _stream()), "embedding")
+
+
+# --------------------------------------------------------------------------- norms
+def add_rmsnorm(h, delta, weight, out, eps: float, rows=None) -> None:
+    """Residual add and RMSNorm in one pass.
+
+    Without ``rows``: h += delta (in place, float), out = norm(h) * weight for every row.
+    With ``rows`` (int32 indices): out[i] = norm(h[rows[i]] + delta[rows[i]]) * weight and
+    h is left as it is.  ``delta`` may be None.
+    """
+    _dev(h, delta, weight, out, rows)
+    _f32(h, "h")
+    hidden = h.shape[-1]
+    _f32(weight, "weight", hidden)
+    n_out = out.shape[0]
+    _need(out.shape[-1] == hidden, "out width differs from h")
+    if delta is not None:
+        _need(delta.shape == h.shape and delta.dtype == out.dtype, "delta must match h's shape and out's type")
+    if rows is None:
+        _need(n_out == h.shape[0], "out must have one row per row of h")
+    else:
+        _i32(rows, "rows", n_out)
+    fn = getattr(library.core(), f"jv_add_rmsnorm_{_suffix(out.dtype)}")
+    _check(
+        fn(_ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), c_int(n_out), c_int(hidden),
+           c_float(eps), _stream()),
+        "add_rmsnorm",
+    )
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out=None) -> torch.Tensor:
+    """RMSNorm over the last axis of a contiguous tensor."""
+    out = torch.empty_like(x) if out is None else out
+    _dev(x, weight, out)
+    n = x.shape[-1]
+    _f32(weight, "weight", n)
+    _need(out.shape == x.shape and out.dtype == x.dtype, "out must match x")
+    fn = getattr(library.core(), f"jv_rmsnorm_{_suffix(x.dtype)}")
+    _check(fn(_ptr(out), _ptr(x), _ptr(weight), c_longlong(x.numel() // n), c_int(n), c_float(eps), _stream()),
+           "rmsnorm")
+    return out
+
+
+def cast_rows(x: torch.Tensor, dtype: torch.dtype, rows=None) -> torch.Tensor:
+    """Copy (selected) rows of a float matrix into a new matrix of ``dtype``."""
+    _dev(x, rows)
+    _f32(x, "x")
+    n_out = x.shape[0] if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, "rows")
+    out = torch.empty((n_out, x.shape[1]), dtype=dtype, device=x.device)
+    fn = getattr(library.core(), f"jv_cast_rows_{_suffix(dtype)}")
+    _check(fn(_ptr(out), _ptr(x), _ptr(rows), c_int(n_out), c_int(x.shape[1]), _stream()), "cast_rows")
+    return out
+
+
+# --------------------------------------------------------------------------- activation
+def silu_mul(gate_up: torch.Tensor, out=None) -> torch.Tensor:
+    """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j] for gate_up of width 2 I."""
+    _dev(gate_up)
+    n, two_i = gate_up.shape
+    _need(two_i % 2 == 0, "gate_up must have an even width")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((n, inter), dtype=gate_up.dtype, device=gate_up.device)
+    _dev(out)
+    _need(out.shape == (n, inter) and out.dtype == gate_up.dtype, "out must be [tokens, I] of gate_up's type")
+    fn = getattr(library.core(), f"jv_silu_mul_{_suffix(gate_up.dtype)}")
+    _check(fn(_ptr(out), _ptr(gate_up), c_longlong(n), c_int(inter), _stream()), "silu_mul")
+    return out
+
+
+# --------------------------------------------------------------------------- attention input
+def qk_norm_rope_write(qkv, positions, slot_mapping, q_weight, k_weight, eps, inv_freq, rotary_dim,
+                       interleaved, k_pages, v_pages, page_size, nq, nkv, head_dim) -> None:
+    """Per-head q/k RMSNorm (if weights given), rotation (if inv_freq given), q in place,
+    k and v into their pages (if pages given).  Cache pages are [pages, nkv, page_size, D]."""
+    _dev(qkv, positions, slot_mapping, q_weight, k_weight, inv_freq, k_pages, v_pages)
+    n = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.shape[1] == (nq + 2 * nkv) * head_dim, "qkv must be [tokens, (nq + 2 nkv) * D]")
+    _i32(positions, "positions", n)
+    _need(head_dim <= 512, "head size above 512 is not supported by the rotation kernel")
+    if q_weight is not None:
+        _f32(q_weight, "q_weight", head_dim)
+    if k_weight is not None:
+        _f32(k_weight, "k_weight", head_dim)
+    if inv_freq is not None:
+        _need(rotary_dim % 2 == 0 and 0 < rotary_dim <= head_dim, "rotary_dim must be even and at most D")
+        _f32(inv_freq, "inv_freq", rotary_dim // 2)
+    if k_pages is not None:
+        _i32(slot_mapping, "slot_mapping", n)
+        for p in (k_pages, v_pages):
+            _need(p.dtype == qkv.dtype and p.dim() == 4 and tuple(p.shape[1:]) == (nkv, page_size, head_dim),
+                  "cache pages must be [pages, nkv, page_size, D] of the activation type")
+    fn = getattr(library.core(), f"jv_qk_norm_rope_write_{_suffix(qkv.dtype)}")
+    _check(
+        fn(_ptr(qkv), _ptr(positions), _ptr(slot_mapping if k_pages is not None else None), _ptr(q_weight),
+           _ptr(k_weight), c_float(eps), _ptr(inv_freq), c_int(rotary_dim if inv_freq is not None else 0),
+           c_int(1 if interleaved else 0), _ptr(k_pages), _ptr(v_pages), c_int(page_size), c_int(n),
+           c_int(nq), c_int(nkv), c_int(head_dim), _stream()),
+        "qk_norm_rope_write",
+    )
+
+
+# --------------------------------------------------------------------------- attention
+def paged_attention_generic(out, q, q_row_stride, k_pages, v_pages, block_tables, token_req, positions,
+                            nq, nkv, head_dim, scale, window=0) -> None:
+    """Causal attention of every token over its request's pages (generic float-math kernel).
+
+    ``q`` is any tensor whose row t holds the q heads at [t * q_row_stride + h * D]."""
+    _dev(out, q, k_pages, v_pages, block_tables, token_req, positions)
+    n = out.shape[0]
+    _need(out.shape == (n, nq * head_dim) and out.dtype == q.dtype, "out must be [tokens, nq * D] of q's type")
+    _need(q.numel() >= (n - 1) * q_row_stride + nq * head_dim if n else True, "q is too small for its stride")
+    _need(nkv > 0 and nq % nkv == 0, "q heads must be a multiple of kv heads")
+    _need(head_dim <= 512, "head size above 512 is not supported")
+    page_size = k_pages.shape[2]
+    for p in (k_pages, v_pages):
+        _need(p.dtype == q.dtype and p.dim() == 4 and tuple(p.shape[1:]) == (nkv, page_size, head_dim),
+              "cache pages must be [pages, nkv, page_size, D] of q's type")
+    _need(block_tables.dim() == 2, "block_tables must be [requests, pages]")
+    _i32(block_tables, "block_tables")
+    _i32(token_req, "token_req", n)
+    _i32(positions, "positions", n)
+    fn = getattr(library.core(), f"jv_paged_attention_generic_{_suffix(q.dtype)}")
+    _check(
+        fn(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages), _ptr(block_tables),
+           c_int(block_tables.shape[1]), _ptr(token_req), _ptr(positions), c_int(page_size), c_int(n),
+           c_int(nq), c_int(nkv), c_int(head_dim), c_float(scale), c_int(window or 0), _stream()),
+        "paged_attention_generic",
+    )
+
+
+# --------------------------------------------------------------------------- matrix products
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, out=None) -> torch.Tensor:
+    """out = a @ w.T in true 32-bit (float FMA).  a [M, K], w [N, K], both row-major."""
+    _dev(a, w)
+    _f32(a, "a")
+    _f32(w, "w")
+    m, k = a.shape
+    n = w.shape[0]
+    _need(w.shape[1] == k, f"inner sizes differ: {k} and {w.shape[1]}")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    _dev(out)
+    _need(out.shape == (m, n) and out.dtype == torch.float32, "out must be float32 [M, N]")
+    fn = library.core().jv_gemm_f32
+    _check(fn(_ptr(out), _ptr(a), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(k), c_longlong(k),
+              c_longlong(n), _stream()), "gemm_f32")
+    return out
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:
+    """x @ w.T for w stored [out, in].
+
+    float32: the library's own float-FMA kernel (no reduced-precision matrix mode).
+    bfloat16: a plain library matrix product (hipBLASLt through torch), float accumulation.
+    """
+    if x.dtype == torch.float32:
+        y = gemm_f32(x, w)
+    else:
+        _need(x.dtype == w.dtype, "x and w must have one type")
+        y = torch.mm(x, w.t())
+    if out_dtype is not None and y.dtype != out_dtype:
+        y = y.to(out_dtype)
+    return y
+
+
+# --------------------------------------------------------------------------- sampling
+def sample(logits: torch.Tensor, temperature=None, keys=None, out=None) -> torch.Tensor:
+    """One token per row of float logits.  temperature[r] <= 0 (or None): greedy, lowest
+    index among maxima; otherwise a draw from softmax(logits / temperature[r]) that depends
+    on keys[r] (int64) and the row's logits only."""
+    _dev(logits, temperature, keys)
+    _f32(logits, "logits")
+    m, v = logits.shape
+    if temperature is not None:
+        _f32(temperature, "temperature", m)
+        _need(keys is not None and keys.dtype == torch.int64 and keys.numel() == m, "keys must be int64, one per row")
+    if out is None:
+        out = torch.empty((m,), dtype=torch.int32, device=logits.device)
+    fn = library.core().jv_sample
+    _check(fn(_ptr(out), _ptr(logits), c_longlong(v), c_int(m), c_int(v), _ptr(temperature),
+              _ptr(keys if temperature is not None else None), _stream()), "sample")
+    return out

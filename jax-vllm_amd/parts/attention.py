@@ -1,0 +1,85 @@
+"""Grouped-query causal attention over a paged cache: the token mixer of Qwen3.
+
+Reference: ``jllm/model/common.py:114-137`` (projections, head layout, output
+projection), ``:107-111`` (optional per-head q/k RMSNorm before the rotation),
+``:173-214`` (scores, mask, softmax, kv head = q head // group).  The three input
+projections are one matrix product against the row-concatenated weight; scores,
+mask and softmax are float inside the attention kernels; keys are stored after
+norm and rotation, values as projected (``jllm/engine/generate.py:54-59``).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from ..ops import kernels as K
+from .spec import KVCacheSpec, LayerMemory, PartSpec, StepContext, TensorSpec, build_part, register_part
+
+
+class GroupedQueryAttention:
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 qk_norm_eps: Optional[float] = None, position: Optional[PartSpec] = None,
+                 window: Optional[int] = None, scale: Optional[float] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} q heads are not a multiple of {num_kv_heads} kv heads")
+        self.hidden_size, self.nq, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
+        self.qk_norm_eps = qk_norm_eps
+        self.window = int(window) if window else None
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
+        self.position = build_part("position", position) if position is not None else None
+        self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+
+    # ---- declarations
+    def tensors(self) -> dict:
+        t = {
+            "q_proj.weight": TensorSpec((self.nq * self.d, self.hidden_size)),
+            "k_proj.weight": TensorSpec((self.nkv * self.d, self.hidden_size)),
+            "v_proj.weight": TensorSpec((self.nkv * self.d, self.hidden_size)),
+            "o_proj.weight": TensorSpec((self.hidden_size, self.nq * self.d)),
+        }
+        if self.qk_norm_eps is not None:
+            t["q_norm.weight"] = TensorSpec((self.d,), role="vector", init="norm")
+            t["k_norm.weight"] = TensorSpec((self.d,), role="vector", init="norm")
+        return t
+
+    def cache_spec(self) -> Optional[KVCacheSpec]:
+        return KVCacheSpec(self.nkv, self.d, self.window)
+
+    def state_spec(self):
+        return None
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        self.dtype = dtype
+        self.w_qkv = torch.cat(
+            [tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0
+        ).contiguous()
+        self.w_o = tensors["o_proj.weight"]
+        if self.qk_norm_eps is not None:
+            self.q_norm, self.k_norm = tensors["q_norm.weight"], tensors["k_norm.weight"]
+        if self.position is not None:
+            self.position.bind({}, dtype, self.w_o.device)
+
+    # ---- one step
+    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
+        n = x.shape[0]
+        qkv = K.linear(x, self.w_qkv)
+        inv_freq, rotary_dim, interleaved = (
+            self.position.fused_arguments() if self.position is not None else (None, 0, False)
+        )
+        writes = mem.writes
+        K.qk_norm_rope_write(
+            qkv, ctx.positions, ctx.slot_mappings[mem.group] if writes else None, self.q_norm, self.k_norm,
+            self.qk_norm_eps or 0.0, inv_freq, rotary_dim, interleaved,
+            mem.k_pages if writes else None, mem.v_pages if writes else None, ctx.page_size,
+            self.nq, self.nkv, self.d,
+        )
+        out = torch.empty((n, self.nq * self.d), dtype=x.dtype, device=x.device)
+        from . import attention_backend
+
+        attention_backend.run(self, out, qkv, ctx, mem)
+        return K.linear(out, self.w_o)
+
+
+register_part("mixer", "gqa_attention", GroupedQueryAttention)

@@ -1,0 +1,47 @@
+"""Token embedding and output head.  Reference: ``jllm/model/common.py:35-41`` (row gather,
+``x @ W.T`` without bias) and ``jllm/model/weights.py:143-146`` (a tied head is the
+embedding table itself, one buffer)."""
+from __future__ import annotations
+
+import torch
+
+from ..ops import kernels as K
+from .spec import TensorSpec, register_part
+
+
+class TokenEmbedding:
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.weight = None
+
+    def tensors(self) -> dict:
+        return {"weight": TensorSpec((self.vocab_size, self.hidden_size))}
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        self.weight = tensors["weight"]
+
+    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+        """Float residual stream [tokens, hidden] of the rows ``ids`` (int32, already range-checked)."""
+        h = torch.empty((ids.numel(), self.hidden_size), dtype=torch.float32, device=ids.device)
+        K.embedding(h, self.weight, ids)
+        return h
+
+
+class LinearHead:
+    def __init__(self, vocab_size: int, hidden_size: int):
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.weight = None
+
+    def tensors(self) -> dict:
+        return {"weight": TensorSpec((self.vocab_size, self.hidden_size))}
+
+    def bind(self, tensors: dict, dtype: torch.dtype) -> None:
+        self.weight = tensors["weight"]
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """Float logits [rows, vocab]."""
+        return K.linear(x, self.weight, out_dtype=torch.float32)
+
+
+register_part("embedding", "token_embedding", TokenEmbedding)
+register_part("head", "linear_head", LinearHead)

@@ -1,0 +1,41 @@
+"""Token choice above the step function.
+
+Greedy: argmax of the float logits, lowest index on ties (reference:
+``jllm/engine/generate.py:142``, ``jllm/engine/state.py:66``; it is the only rule the
+reference has).  Temperature: a draw from ``softmax(logits / T)`` computed in float.  The
+draw of a request's k-th token depends on (seed, request, k) and that token's logits only,
+so it is the same under any batching, cutting or recomputation.
+"""
+from __future__ import annotations
+
+import hashlib
+from typing import Sequence
+
+import torch
+
+from ..ops import kernels as K
+
+
+def draw_key(seed: int, request_key: int, index: int) -> int:
+    """64-bit key (as a signed int64 value) of one draw."""
+    d = hashlib.blake2b(f"{seed}:{request_key}:{index}".encode(), digest_size=8).digest()
+    v = int.from_bytes(d, "little")
+    return v - (1 << 64) if v >= (1 << 63) else v
+
+
+class Sampler:
+    def __init__(self, device):
+        self.device = device
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], keys: Sequence[int]) -> list:
+        """One token id per row of ``logits`` [M, V] (float32, on the device)."""
+        m = logits.shape[0]
+        if m == 0:
+            return []
+        if all(t <= 0.0 for t in temperatures):
+            out = K.sample(logits)
+        else:
+            temp = torch.tensor(list(temperatures), dtype=torch.float32, device=self.device)
+            key = torch.tensor(list(keys), dtype=torch.int64, device=self.device)
+            out = K.sample(logits, temp, key)
+        return out.tolist()

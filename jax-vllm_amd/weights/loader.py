@@ -1,0 +1,91 @@
+"""Loads a model folder (``config.json`` + ``*.safetensors``) into a bound ``DecoderModel``.
+
+Reference: ``jllm/model/weights.py:21-37`` (all shards in sorted order, a later shard wins
+on a duplicate name, every tensor cast to the engine's type) and ``:161-170`` (the model
+is chosen by ``architectures[0]``).  Unlike the reference, names and shapes are checked
+before anything is copied, and all problems are reported in one error.
+
+Types on the device: tensors of role "matrix" take the compute type (bfloat16 or float32),
+role "vector" is float32 (16-bit values widen exactly, 32-bit values stay as stored),
+role "table" is int32.
+"""
+from __future__ import annotations
+
+from pathlib import Path
+
+import torch
+
+from ..config.registry import resolve
+from ..parts.model import DecoderModel
+from .safetensors_io import open_shards
+
+TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+class WeightsError(ValueError):
+    """The checkpoint does not fit the model: lists missing and unexpected tensors and wrong shapes."""
+
+    def __init__(self, where, missing, unexpected, wrong_shape, wrong_type):
+        self.missing, self.unexpected = sorted(missing), sorted(unexpected)
+        self.wrong_shape, self.wrong_type = sorted(wrong_shape), sorted(wrong_type)
+        lines = [f"checkpoint {where} does not fit the model:"]
+        if self.missing:
+            lines.append(f"  missing tensors ({len(self.missing)}): " + ", ".join(self.missing))
+        if self.unexpected:
+            lines.append(f"  unexpected tensors ({len(self.unexpected)}): " + ", ".join(self.unexpected))
+        for name, got, want in self.wrong_shape:
+            lines.append(f"  wrong shape: {name} is {list(got)}, the model needs {list(want)}")
+        for name, got, want in self.wrong_type:
+            lines.append(f"  wrong type: {name} is stored as {got}, the model needs {want} data")
+        super().__init__("\n".join(lines))
+
+
+def target_dtype(role: str, compute_dtype: torch.dtype) -> torch.dtype:
+    if role == "matrix":
+        return compute_dtype
+    if role == "vector":
+        return torch.float32
+    if role == "table":
+        return torch.int32
+    raise ValueError(f"unknown tensor role {role!r}")
+
+
+def check_against_specs(where, specs: dict, ignored: set, available: dict) -> None:
+    """``available``: name -> (dtype, shape) found in the checkpoint."""
+    missing = [n for n in specs if n not in available]
+    unexpected = [n for n in available if n not in specs and n not in ignored]
+    wrong_shape, wrong_type = [], []
+    for name, ts in specs.items():
+        if name not in available:
+            continue
+        dtype, shape = available[name]
+        if tuple(shape) != tuple(ts.shape):
+            wrong_shape.append((name, tuple(shape), tuple(ts.shape)))
+        is_float = dtype.is_floating_point
+        if (ts.role == "table") == is_float:
+            wrong_type.append((name, str(dtype).replace("torch.", ""), "integer" if ts.role == "table" else "floating"))
+    if missing or unexpected or wrong_shape or wrong_type:
+        raise WeightsError(where, missing, unexpected, wrong_shape, wrong_type)
+
+
+def load_model(folder, dtype: str = "bfloat16", device="cuda") -> tuple:
+    """(bound DecoderModel, typed config) of a model folder."""
+    folder = Path(folder)
+    arch, cfg, _ = resolve(folder)
+    model = DecoderModel(arch.build_spec(cfg))
+    specs, ignored = model.tensor_specs(), model.ignored_tensor_names()
+    compute = TORCH_DTYPES[dtype]
+    shards = list(open_shards(folder))
+    owner, available = {}, {}
+    for shard in shards:  # a later shard wins
+        for name, entry in shard.entries.items():
+            owner[name], available[name] = shard, entry
+    check_against_specs(folder, specs, ignored, available)
+    tensors = {}
+    for name, ts in specs.items():
+        src = owner[name].tensor(name)
+        tensors[name] = src.to(device).to(target_dtype(ts.role, compute)).contiguous()
+    model.bind(tensors, compute)
+    for shard in shards:
+        shard.close()
+    return model, cfg

@@ -1,0 +1,303 @@
+"""Each HIP kernel alone against a plain torch reference of the same operation, at sizes
+other than the engine's test models (widths and vocabularies that are no power of two,
+head sizes in steps of 16, odd head counts)."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def K():
+    from jax_vllm_amd.ops import kernels
+
+    return kernels
+
+
+def tol(dtype, f32=1e-5, bf16=2e-2):
+    return dict(rtol=f32, atol=f32) if dtype == torch.float32 else dict(rtol=bf16, atol=bf16)
+
+
+def randn(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden,vocab", [(72, 333), (4096, 1000)])
+def test_embedding(dtype, hidden, vocab):
+    table = randn(vocab, hidden, dtype=dtype)
+    ids = torch.tensor([0, vocab - 1, 5, 5, 17], dtype=torch.int32).cuda()
+    h = torch.empty(5, hidden, dtype=torch.float32).cuda()
+    K().embedding(h, table, ids)
+    torch.testing.assert_close(h, table[ids.long()].float(), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden", [80, 1000, 4096])
+def test_add_rmsnorm(dtype, hidden):
+    n, eps = 7, 1e-5
+    h = randn(n, hidden, seed=1)
+    delta = randn(n, hidden, dtype=dtype, seed=2)
+    w = 1 + 0.1 * randn(hidden, seed=3)
+    h0 = h.clone()
+    out = torch.empty(n, hidden, dtype=dtype).cuda()
+    K().add_rmsnorm(h, delta, w, out, eps)
+    x = h0 + delta.float()
+    ref = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + eps) * w
+    torch.testing.assert_close(h, x, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(out.float(), ref, **tol(dtype))
+    # first layer: no delta, h untouched
+    h1 = h0.clone()
+    K().add_rmsnorm(h1, None, w, out, eps)
+    torch.testing.assert_close(h1, h0, rtol=0, atol=0)
+    ref1 = h0 * torch.rsqrt((h0 * h0).mean(-1, keepdim=True) + eps) * w
+    torch.testing.assert_close(out.float(), ref1, **tol(dtype))
+    # selected rows: h untouched, sum redone on the fly
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32).cuda()
+    h2 = h0.clone()
+    out2 = torch.empty(3, hidden, dtype=dtype).cuda()
+    K().add_rmsnorm(h2, delta, w, out2, eps, rows)
+    torch.testing.assert_close(h2, h0, rtol=0, atol=0)
+    torch.testing.assert_close(out2.float(), ref[rows.long()], **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rmsnorm_last_axis(dtype):
+    x = randn(5, 3, 48, dtype=dtype, seed=4)
+    w = 1 + 0.2 * randn(48, seed=5)
+    out = K().rmsnorm(x, w, 1e-6)
+    xf = x.float()
+    ref = xf * torch.rsqrt((xf * xf).mean(-1, keepdim=True) + 1e-6) * w
+    torch.testing.assert_close(out.float(), ref, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("inter", [176, 12288])
+def test_silu_mul(dtype, inter):
+    gu = randn(9, 2 * inter, dtype=dtype, seed=6, scale=3.0)
+    out = K().silu_mul(gu)
+    g, u = gu.float()[:, :inter], gu.float()[:, inter:]
+    torch.testing.assert_close(out.float(), torch.nn.functional.silu(g) * u, **tol(dtype))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 50, 70), (5, 333, 80), (70, 130, 257), (130, 64, 16)])
+def test_gemm_f32_is_true_32bit(m, n, k):
+    a, w = randn(m, k, seed=7), randn(n, k, seed=8)
+    out = K().gemm_f32(a, w)
+    ref = (a.double() @ w.double().T)
+    # float accumulation over k terms: error far below any 16- or 19-bit matrix mode (~1e-3)
+    torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=1e-5 * math.sqrt(k))
+    # a row's result does not depend on the other rows of the batch
+    if m > 1:
+        single = K().gemm_f32(a[:1].contiguous(), w)
+        torch.testing.assert_close(single, out[:1], rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 96, 64), (8, 224, 96), (33, 512, 96)])
+def test_linear_bf16(m, n, k):
+    a, w = randn(m, k, dtype=torch.bfloat16, seed=9), randn(n, k, dtype=torch.bfloat16, seed=10)
+    out = K().linear(a, w)
+    ref = a.float() @ w.float().T
+    torch.testing.assert_close(out.float(), ref, rtol=2e-2, atol=2e-2 * math.sqrt(k) / 8)
+
+
+# ------------------------------------------------------------------ q/k norm + rotation + page write
+def rope_reference(x, pos, inv_freq, rotary_dim, interleaved):
+    """x [T, heads, D] float; rotation of the first rotary_dim elements of each head."""
+    ang = pos.float()[:, None] * inv_freq[None, :]
+    cos, sin = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    out = x.clone()
+    half = rotary_dim // 2
+    if interleaved:
+        a, b = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+        out[..., 0:rotary_dim:2] = a * cos - b * sin
+        out[..., 1:rotary_dim:2] = b * cos + a * sin
+    else:
+        a, b = x[..., :half], x[..., half:rotary_dim]
+        out[..., :half] = a * cos - b * sin
+        out[..., half:rotary_dim] = b * cos + a * sin
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nq,nkv,d,rotary_dim,interleaved,with_norm",
+                         [(4, 2, 16, 16, False, True), (5, 5, 48, 48, False, True), (6, 2, 128, 128, False, True),
+                          (3, 1, 80, 32, False, False), (4, 4, 32, 32, True, True), (8, 2, 256, 64, True, False)])
+def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_norm):
+    t, page_size, pages, eps = 11, 4, 9, 1e-5
+    qkv = randn(t, (nq + 2 * nkv) * d, dtype=dtype, seed=11)
+    pos = torch.tensor([0, 1, 2, 3, 100, 101, 4095, 7, 8, 9, 31999], dtype=torch.int32).cuda()
+    slots = torch.tensor([4, 5, 6, 7, 32, 33, 12, -1, 20, 21, 35], dtype=torch.int32).cuda()
+    qw = (1 + 0.1 * randn(d, seed=12)) if with_norm else None
+    kw = (1 + 0.1 * randn(d, seed=13)) if with_norm else None
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))).cuda()
+    k_pages = torch.zeros(pages, nkv, page_size, d, dtype=dtype).cuda()
+    v_pages = torch.zeros_like(k_pages)
+    x = qkv.float().view(t, nq + 2 * nkv, d).clone()
+    K().qk_norm_rope_write(qkv, pos, slots, qw, kw, eps, inv_freq, rotary_dim, interleaved, k_pages, v_pages,
+                           page_size, nq, nkv, d)
+    q, k, v = x[:, :nq], x[:, nq:nq + nkv], x[:, nq + nkv:]
+    if with_norm:
+        q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * qw
+        k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * kw
+    q = rope_reference(q, pos, inv_freq, rotary_dim, interleaved)
+    k = rope_reference(k, pos, inv_freq, rotary_dim, interleaved)
+    got_q = qkv.float().view(t, nq + 2 * nkv, d)[:, :nq]
+    # large positions: the angle itself carries float rounding (pos * inv_freq ~ 3e4 * 1 has ulp 2e-3)
+    big = dict(rtol=1e-2, atol=1e-2) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    small = tol(dtype, f32=2e-5, bf16=2e-2)
+    near = pos.cpu() < 200
+    torch.testing.assert_close(got_q[near.cuda()], q[near.cuda()], **small)
+    torch.testing.assert_close(got_q, q, **big)
+    exp_k = torch.zeros(pages, nkv, page_size, d).cuda()
+    exp_v = torch.zeros_like(exp_k)
+    for i, s in enumerate(slots.tolist()):
+        if s >= 0:
+            exp_k[s // page_size, :, s % page_size] = k[i]
+            exp_v[s // page_size, :, s % page_size] = v[i]
+    torch.testing.assert_close(k_pages.float(), exp_k, **big)
+    torch.testing.assert_close(v_pages.float(), exp_v, rtol=0, atol=0)  # values are copied untouched
+    written = torch.zeros(pages * page_size, dtype=torch.bool)
+    written[[s for s in slots.tolist() if s >= 0]] = True
+    untouched = ~written.view(pages, page_size).cuda()
+    assert (k_pages.float().abs().sum((1, 3))[untouched] == 0).all()  # nothing beside the named slots
+
+
+# ------------------------------------------------------------------ paged attention
+def build_paged(k, v, page_size, seed=0, extra_pages=3):
+    """Scatter per-request [T, nkv, D] keys/values over shuffled pages; returns pages and tables."""
+    g = torch.Generator().manual_seed(seed)
+    need = [-(-kk.shape[0] // page_size) for kk in k]
+    total = sum(need) + extra_pages + 1
+    order = (torch.randperm(total - 1, generator=g) + 1).tolist()
+    nkv, d = k[0].shape[1], k[0].shape[2]
+    k_pages = torch.randn(total, nkv, page_size, d, generator=g) * 50  # garbage where no key lives
+    v_pages = torch.randn(total, nkv, page_size, d, generator=g) * 50
+    tables = torch.zeros(len(k), max(need), dtype=torch.int32)
+    for r, (kk, vv) in enumerate(zip(k, v)):
+        for p in range(need[r]):
+            page = order.pop()
+            tables[r, p] = page
+            chunk = slice(p * page_size, min((p + 1) * page_size, kk.shape[0]))
+            n = chunk.stop - chunk.start
+            k_pages[page, :, :n] = kk[chunk].transpose(0, 1)
+            v_pages[page, :, :n] = vv[chunk].transpose(0, 1)
+    return k_pages, v_pages, tables
+
+
+def attention_reference(q, k, v, positions, scale, window=None):
+    """q [Tq, nq, D] at absolute ``positions``; k, v [Tk, nkv, D]; float64."""
+    nq, nkv = q.shape[1], k.shape[1]
+    kk = torch.repeat_interleave(k.double(), nq // nkv, dim=1)
+    vv = torch.repeat_interleave(v.double(), nq // nkv, dim=1)
+    s = torch.einsum("qhd,khd->hqk", q.double(), kk) * scale
+    j = torch.arange(k.shape[0])[None, :]
+    p = positions[:, None]
+    mask = j <= p
+    if window:
+        mask &= j > p - window
+    s = s.masked_fill(~mask[None], float("-inf"))
+    return torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), vv)
+
+
+ATT_CASES = [
+    # nq, nkv, d, page_size, [(context_len, q_len)], window
+    (4, 2, 16, 8, [(0, 5), (0, 17), (0, 33)], None),
+    (6, 2, 32, 16, [(0, 1), (9, 1), (40, 24), (0, 64), (100, 1)], None),
+    (5, 5, 48, 32, [(37, 2), (0, 70)], None),
+    (8, 2, 128, 16, [(300, 1), (0, 130), (255, 3)], None),
+    (3, 1, 80, 4, [(20, 9), (3, 1)], None),
+    (4, 2, 64, 16, [(50, 10), (0, 40), (200, 1)], 24),
+    (16, 2, 256, 16, [(10, 3)], None),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", ATT_CASES, ids=[f"h{c[0]}g{c[1]}d{c[2]}p{c[3]}w{c[5]}" for c in ATT_CASES])
+def test_paged_attention_generic(dtype, case):
+    nq, nkv, d, page_size, reqs, window = case
+    scale = 1.0 / math.sqrt(d)
+    g = torch.Generator().manual_seed(5)
+    ks = [torch.randn(c + q, nkv, d, generator=g).to(dtype).float() for c, q in reqs]
+    vs = [torch.randn(c + q, nkv, d, generator=g).to(dtype).float() for c, q in reqs]
+    qs = [torch.randn(q, nq, d, generator=g).to(dtype).float() for c, q in reqs]
+    k_pages, v_pages, tables = build_paged(ks, vs, page_size)
+    n = sum(q for _, q in reqs)
+    # q rows live inside a fused qkv-like buffer: row stride larger than nq * d
+    stride = (nq + 2 * nkv) * d
+    qbuf = torch.zeros(n, stride)
+    positions, token_req, refs, at = [], [], [], 0
+    for r, (c, ql) in enumerate(reqs):
+        qbuf[at:at + ql, :nq * d] = qs[r].reshape(ql, nq * d)
+        pos = torch.arange(c, c + ql)
+        positions += pos.tolist()
+        token_req += [r] * ql
+        refs.append(attention_reference(qs[r], ks[r], vs[r], pos, scale, window))
+        at += ql
+    ref = torch.cat(refs).reshape(n, nq * d)
+    out = torch.empty(n, nq * d, dtype=dtype).cuda()
+    K().paged_attention_generic(
+        out, qbuf.to(dtype).cuda(), stride, k_pages.to(dtype).cuda(), v_pages.to(dtype).cuda(), tables.cuda(),
+        torch.tensor(token_req, dtype=torch.int32).cuda(), torch.tensor(positions, dtype=torch.int32).cuda(),
+        nq, nkv, d, scale, window or 0)
+    torch.testing.assert_close(out.double().cpu(), ref, **tol(dtype, f32=2e-5, bf16=2e-2))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("far_key", [0, 15, 16, 17, 255, 256, 511, 640])
+def test_attention_finds_one_far_key(dtype, far_key):
+    """One key among hundreds is made to dominate: the output must be that key's value, wherever
+    in its page (first slot, last slot) and however far back it lies."""
+    nq, nkv, d, page_size, ctx = 4, 2, 64, 16, 641
+    g = torch.Generator().manual_seed(far_key)
+    k = torch.randn(ctx, nkv, d, generator=g) * 0.1
+    v = torch.randn(ctx, nkv, d, generator=g)
+    q = torch.randn(1, nq, d, generator=g) * 0.1
+    q[0, :, 0] = 40.0
+    k[far_key, :, 0] = 40.0          # score 1600/8 = 200 above the rest
+    k_pages, v_pages, tables = build_paged([k], [v], page_size, seed=far_key)
+    out = torch.empty(1, nq * d, dtype=dtype).cuda()
+    K().paged_attention_generic(
+        out, q.reshape(1, -1).to(dtype).cuda(), nq * d, k_pages.to(dtype).cuda(), v_pages.to(dtype).cuda(),
+        tables.cuda(), torch.zeros(1, dtype=torch.int32).cuda(), torch.tensor([ctx - 1], dtype=torch.int32).cuda(),
+        nq, nkv, d, 1.0 / math.sqrt(d))
+    expect = torch.repeat_interleave(v[far_key].to(dtype).float(), nq // nkv, dim=0).reshape(1, -1)
+    torch.testing.assert_close(out.float().cpu(), expect, rtol=1e-3, atol=1e-3)
+
+
+# ------------------------------------------------------------------ sampling
+def test_greedy_is_argmax_lowest_index_on_ties():
+    logits = randn(6, 777, seed=20)
+    logits[2, 100] = logits[2, 500] = 99.0
+    logits[4, 776] = 50.0
+    out = K().sample(logits)
+    ref = torch.argmax(logits, dim=-1)
+    assert out.tolist()[:2] == ref.tolist()[:2]
+    assert out[2].item() == 100 and out[4].item() == 776
+
+
+def test_temperature_sampling_matches_softmax():
+    v, n, temp = 11, 20000, 0.8
+    logits1 = randn(1, v, seed=21, scale=1.5)
+    logits = logits1.expand(n, v).contiguous()
+    keys = torch.arange(n, dtype=torch.int64).cuda() * 7919 + 3
+    t = torch.full((n,), temp, dtype=torch.float32).cuda()
+    out = K().sample(logits, t, keys)
+    freq = torch.bincount(out.long().cpu(), minlength=v).double() / n
+    p = torch.softmax(logits1[0].double().cpu() / temp, -1)
+    # binomial standard deviation of a frequency is at most 0.5 / sqrt(n) = 0.0035
+    assert (freq - p).abs().max().item() < 0.015
+    # the draw depends on key and logits only: same keys in another order, another batch size
+    perm = torch.randperm(n)[:100].cuda()
+    out2 = K().sample(logits[perm].contiguous(), t[:100].contiguous(), keys[perm].contiguous())
+    assert out2.tolist() == out[perm].tolist()
+    # temperature 0 rows beside sampled rows are greedy
+    t2 = t.clone()
+    t2[::2] = 0.0
+    out3 = K().sample(logits, t2, keys)
+    assert (out3[::2] == torch.argmax(logits1[0])).all()
+    assert out3[1::2].tolist() == out[1::2].tolist()

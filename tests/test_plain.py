@@ -1,0 +1,220 @@
+"""Pins the plain implementation by what fixes it beside the reference's text:
+library routines it must reduce to, invariants, and the reference's own vectors."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.plain import qwen3_plain as P
+from tests.tiny import TINY_A, TINY_B, make_weights_dict
+
+
+def test_rms_norm_is_library_rms_norm():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(5, 7, 24, generator=g)
+    w = 1 + 0.1 * torch.randn(24, generator=g)
+    ref = F.rms_norm(x, (24,), w, 1e-5)
+    torch.testing.assert_close(P.rms_norm(w, 1e-5, x), ref, rtol=1e-6, atol=1e-6)
+
+
+def test_rms_norm_invariants():
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(3, 40, generator=g)
+    y = P.rms_norm(torch.ones(40), 0.0, x)
+    torch.testing.assert_close((y * y).mean(-1), torch.ones(3), rtol=1e-5, atol=1e-5)
+    # scale invariance (a norm applied after the weight, or a mean instead of a mean square, breaks it)
+    torch.testing.assert_close(P.rms_norm(torch.ones(40), 0.0, 7.5 * x), y, rtol=1e-5, atol=1e-5)
+    # eps sits inside the square root, next to the mean square
+    z = P.rms_norm(torch.ones(40), 3.0, x)
+    torch.testing.assert_close(z, x / torch.sqrt((x * x).mean(-1, keepdim=True) + 3.0))
+
+
+def test_rope_position_zero_is_identity_and_pairs_are_rotated():
+    d = 16
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 5, d, generator=g)
+    pos = torch.tensor([0, 1, 7, 100, 4095])
+    cos, sin = P.rope_cos_sin(d, 10000.0, pos, torch.float32)
+    y = P.apply_rope(x, cos, sin)
+    torch.testing.assert_close(y[:, 0], x[:, 0])
+    # element i pairs with i + d/2: each such pair keeps its length (pairing (2i, 2i+1) fails this)
+    n_in = x[..., : d // 2] ** 2 + x[..., d // 2 :] ** 2
+    n_out = y[..., : d // 2] ** 2 + y[..., d // 2 :] ** 2
+    torch.testing.assert_close(n_in, n_out, rtol=1e-4, atol=1e-5)
+    # the pair (i, i+d/2) turns by pos * theta^(-2i/d), counter-clockwise
+    i = 3
+    ang = 7 * 10000.0 ** (-2 * i / d)
+    a, b = x[0, 2, i], x[0, 2, i + d // 2]
+    assert y[0, 2, i].item() == pytest.approx(a * math.cos(ang) - b * math.sin(ang), abs=1e-5)
+    assert y[0, 2, i + d // 2].item() == pytest.approx(b * math.cos(ang) + a * math.sin(ang), abs=1e-5)
+
+
+def test_rope_scores_depend_on_distance_only():
+    d = 32
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(1, 1, d, generator=g)
+    k = torch.randn(1, 1, d, generator=g)
+
+    def score(m, n):
+        cq, sq = P.rope_cos_sin(d, 1e6, torch.tensor([m]), torch.float64)
+        ck, sk = P.rope_cos_sin(d, 1e6, torch.tensor([n]), torch.float64)
+        return (P.apply_rope(q.double(), cq, sq) * P.apply_rope(k.double(), ck, sk)).sum().item()
+
+    assert score(5, 2) == pytest.approx(score(105, 102), abs=1e-4)
+    assert score(5, 2) != pytest.approx(score(5, 3), abs=1e-3)
+
+
+def test_attention_is_library_sdpa_with_gqa():
+    g = torch.Generator().manual_seed(4)
+    nq, nkv, t, d = 6, 2, 9, 8
+    q = torch.randn(nq, t, d, generator=g)
+    k = torch.randn(nkv, t, d, generator=g)
+    v = torch.randn(nkv, t, d, generator=g)
+    ref = F.scaled_dot_product_attention(q[None], k[None], v[None], is_causal=True, enable_gqa=True)[0]
+    torch.testing.assert_close(P.attention_core(q, k, v, P.causal_mask(t, t)), ref, rtol=1e-5, atol=1e-5)
+
+
+def test_attention_without_mask_or_rotation_one_head_is_softmax_formula():
+    g = torch.Generator().manual_seed(5)
+    q = torch.randn(1, 4, 8, generator=g)
+    k = torch.randn(1, 6, 8, generator=g)
+    v = torch.randn(1, 6, 8, generator=g)
+    ref = torch.softmax(q[0] @ k[0].T / math.sqrt(8), -1) @ v[0]
+    out = P.attention_core(q, k, v, torch.ones(4, 6, dtype=torch.bool))
+    torch.testing.assert_close(out[0], ref, rtol=1e-5, atol=1e-6)
+
+
+def test_attention_gqa_head_map_and_single_key():
+    # kv heads made distinguishable: v of kv head j is the constant j+1
+    nq, nkv, t, d = 6, 2, 4, 4
+    g = torch.Generator().manual_seed(6)
+    q = torch.randn(nq, t, d, generator=g)
+    k = torch.randn(nkv, t, d, generator=g)
+    v = torch.stack([torch.full((t, d), float(j + 1)) for j in range(nkv)])
+    out = P.attention_core(q, k, v, P.causal_mask(t, t))
+    for h in range(nq):
+        torch.testing.assert_close(out[h], torch.full((t, d), float(h // 3 + 1)))
+    # first query sees one key only: output equals that key's value row
+    v2 = torch.randn(nkv, t, d, generator=g)
+    out2 = P.attention_core(q, k, v2, P.causal_mask(t, t))
+    torch.testing.assert_close(out2[4, 0], v2[1, 0])
+    # equal keys: output is the mean of the visible values
+    k_eq = torch.ones(nkv, t, d)
+    out3 = P.attention_core(q, k_eq, v2, P.causal_mask(t, t))
+    torch.testing.assert_close(out3[0, 2], v2[0, :3].mean(0), rtol=1e-5, atol=1e-6)
+
+
+def test_lens_mask_matches_reference_vector():
+    """The reference's own case (tests/test_attention_backend.py:29-61): q [2,4,3,2],
+    k,v [2,2,5,2], q_lens [3,1], k_lens [5,2]; the lens rule gives the explicit mask."""
+    rng = np.random.default_rng(0)
+    q = torch.from_numpy(rng.standard_normal((2, 4, 3, 2), dtype=np.float32))
+    k = torch.from_numpy(rng.standard_normal((2, 2, 5, 2), dtype=np.float32))
+    v = torch.from_numpy(rng.standard_normal((2, 2, 5, 2), dtype=np.float32))
+    for b, (ql, kl) in enumerate([(3, 5), (1, 2)]):
+        out = P.attention_core(q[b, :, :ql], k[b, :, :kl], v[b, :, :kl], P.causal_mask(ql, kl))
+        # explicit: query i of the portion sits at absolute position kl - ql + i
+        for i in range(ql):
+            n_vis = kl - ql + i + 1
+            full = P.attention_core(
+                q[b, :, i : i + 1], k[b, :, :n_vis], v[b, :, :n_vis], torch.ones(1, n_vis, dtype=torch.bool)
+            )
+            torch.testing.assert_close(out[:, i : i + 1], full, rtol=1e-5, atol=1e-5)
+
+
+def test_chunk_with_offset_equals_rows_of_whole():
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn(4, 10, 8, generator=g)
+    k = torch.randn(2, 10, 8, generator=g)
+    v = torch.randn(2, 10, 8, generator=g)
+    whole = P.attention_core(q, k, v, P.causal_mask(10, 10))
+    part = P.attention_core(q[:, 6:9], k[:, :9], v[:, :9], P.causal_mask(3, 9))
+    torch.testing.assert_close(part, whole[:, 6:9], rtol=1e-5, atol=1e-6)
+
+
+def test_swiglu_is_library_silu():
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(3, 12, generator=g)
+    wg, wu, wd = (torch.randn(20, 12, generator=g), torch.randn(20, 12, generator=g), torch.randn(12, 20, generator=g))
+    ref = F.linear(F.silu(F.linear(x, wg)) * F.linear(x, wu), wd)
+    torch.testing.assert_close(P.swiglu(wg, wu, wd, x), ref)
+
+
+@pytest.mark.parametrize("tiny", [TINY_A, TINY_B], ids=["A", "B"])
+def test_qk_norm_is_per_head_and_before_rope(tiny):
+    cfg = P_cfg(tiny)
+    w = make_weights_dict(tiny)
+    g = torch.Generator().manual_seed(9)
+    t, hsz = 6, cfg["hidden_size"]
+    x = torch.randn(t, hsz, generator=g)
+    pos = torch.arange(t)
+    p = "model.layers.0.self_attn"
+    base = P.attention_block(w, p, cfg, x, pos)
+    # scaling one q head's projection rows by a constant must change nothing: the per-head
+    # norm divides it out (a norm over all heads at once, or after RoPE with w != 1, fails)
+    d = cfg["head_dim"]
+    w2 = dict(w)
+    qw = w[f"{p}.q_proj.weight"].clone()
+    qw[d : 2 * d] *= 5.0
+    w2[f"{p}.q_proj.weight"] = qw
+    # (up to eps, which does not scale with the head: hence the absolute slack)
+    torch.testing.assert_close(P.attention_block(w2, p, cfg, x, pos), base, rtol=1e-4, atol=2e-5)
+    # while scaling one *element* inside a head does change it
+    qw3 = w[f"{p}.q_proj.weight"].clone()
+    qw3[d] *= 5.0
+    w3 = dict(w)
+    w3[f"{p}.q_proj.weight"] = qw3
+    assert not torch.allclose(P.attention_block(w3, p, cfg, x, pos), base, rtol=1e-3, atol=1e-4)
+
+
+def P_cfg(tiny):
+    c = dict(tiny["config"])
+    nq = c["num_attention_heads"]
+    return dict(
+        vocab_size=c["vocab_size"], hidden_size=c["hidden_size"], intermediate_size=c["intermediate_size"],
+        num_hidden_layers=c["num_hidden_layers"], num_heads=nq, num_kv_heads=c["num_key_value_heads"],
+        head_dim=c["head_dim"], rms_norm_eps=c["rms_norm_eps"], rope_theta=c["rope_theta"],
+        tie_word_embeddings=c["tie_word_embeddings"],
+    )
+
+
+@pytest.mark.parametrize("tiny", [TINY_A, TINY_B], ids=["A", "B"])
+def test_forward_shift_invariance_and_causality(tiny):
+    cfg = P_cfg(tiny)
+    w = make_weights_dict(tiny)
+    rng = np.random.default_rng(3)
+    ids = rng.integers(0, cfg["vocab_size"], size=21).tolist()
+    base = P.forward(w, cfg, ids)
+    assert base.shape == (21, cfg["vocab_size"])
+    # only distances count: shifting every position leaves the logits alone
+    shifted = P.forward(w, cfg, ids, first_position=37)
+    torch.testing.assert_close(shifted, base, rtol=2e-3, atol=2e-4)
+    # causal: a later token does not change earlier logits
+    ids2 = list(ids)
+    ids2[-1] = (ids2[-1] + 1) % cfg["vocab_size"]
+    torch.testing.assert_close(P.forward(w, cfg, ids2)[:-1], base[:-1])
+    # prefix property: forward of a prefix gives the same rows
+    torch.testing.assert_close(P.forward(w, cfg, ids[:9]), base[:9], rtol=1e-4, atol=1e-5)
+
+
+def test_tied_head_uses_embedding_table():
+    cfg = P_cfg(TINY_A)
+    assert cfg["tie_word_embeddings"]
+    w = make_weights_dict(TINY_A)
+    ids = [1, 2, 3]
+    base = P.forward(w, cfg, ids)
+    w2 = dict(w)
+    w2["lm_head.weight"] = torch.zeros_like(w["model.embed_tokens.weight"])  # must be ignored when tied
+    torch.testing.assert_close(P.forward(w2, cfg, ids), base)
+
+
+def test_greedy_generate_stops_on_eos_and_counts_it():
+    cfg = P_cfg(TINY_A)
+    w = make_weights_dict(TINY_A)
+    out = P.greedy_generate(w, cfg, [5, 6, 7], 6)
+    assert len(out) == 6
+    out2 = P.greedy_generate(w, cfg, [5, 6, 7], 6, eos_id=out[2])
+    first = out.index(out[2])
+    assert out2 == out[: first + 1]
