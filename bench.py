@@ -1,0 +1,169 @@
+"""Measurement of the engine on one MI355X: decode tokens/s at batch 8 (the headline), with
+prefill tokens/s at 2,048 tokens and decode at batch 1 and 64 beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+
+The model has the layer sizes of BASELINE.json ``configs[2]`` (Qwen3-8B shape) with random
+weights drawn on the device; prompts are seeded uniform-random token ids of 1,024 tokens;
+a "step" is one decode step of the whole engine (scheduler, step function, sampling).
+It prints ONE JSON line.  More than one GPU is not supported: it says so and exits with 2.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+QWEN3_8B = dict(
+    architectures=["Qwen3ForCausalLM"], num_hidden_layers=36, hidden_size=4096, num_attention_heads=32,
+    num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
+    rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960,
+)
+PROMPT_LEN = 1024
+MAX_CONTEXT = 8192
+PREFILL_TOKENS = 2048
+
+
+def weight_bytes(cfg, layers, itemsize):
+    h, i, v = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    per_layer = (nq + 2 * nkv) * d * h + h * nq * d + 3 * i * h
+    return (per_layer * layers + v * h) * itemsize, per_layer
+
+
+def sync():
+    import torch
+
+    torch.cuda.synchronize()
+
+
+def measure_decode(llm, batch, steps, warmup, rng, vocab):
+    """Tokens/s of ``steps`` decode steps at ``batch`` after prefilling 1,024-token prompts."""
+    from jax_vllm_amd import SamplingParams
+
+    prompts = [rng.integers(0, vocab, size=PROMPT_LEN).tolist() for _ in range(batch)]
+    sp = SamplingParams(max_new_tokens=warmup + steps + 128)
+    for p in prompts:
+        llm.add_request(p, sp)
+    while any(r.num_remaining > 1 or not r.output_ids for r in llm.scheduler.running) or llm.scheduler.waiting:
+        llm.step()  # prefill, untimed
+    for _ in range(warmup):
+        llm.step()
+    sync()
+    ctx_start = sum(r.num_computed for r in llm.scheduler.running) / batch
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ev = llm.step()
+        assert len(ev) == batch
+    sync()
+    dt = time.perf_counter() - t0
+    llm.abort_all()
+    mean_ctx = ctx_start + (steps - 1) / 2.0
+    return batch * steps / dt, dt / steps, mean_ctx
+
+
+def measure_prefill(llm, rng, vocab, repeats=3):
+    from jax_vllm_amd.engine.core import StepEntry
+
+    core = llm.core
+    best = None
+    for i in range(repeats + 1):
+        toks = rng.integers(0, vocab, size=PREFILL_TOKENS).tolist()
+        rid = f"prefill{i}"
+        core.start_request(rid)
+        sync()
+        t0 = time.perf_counter()
+        core.run([StepEntry(rid, toks, [PREFILL_TOKENS - 1])])
+        sync()
+        dt = time.perf_counter() - t0
+        core.finish_request(rid)
+        if i > 0:  # the first run warms up
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
+                    help="run only the first layers of the 36 (reported in config)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--skip-points", action="store_true", help="measure the headline batch only")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from jax_vllm_amd import LLM
+
+    cfg = dict(QWEN3_8B)
+    layers = args.layers
+    cfg["num_hidden_layers"] = layers
+    vocab = cfg["vocab_size"]
+    rng = np.random.default_rng(0)
+    max_batch = args.batch if args.skip_points else max(64, args.batch)
+    block = 16
+    llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=max_batch,
+              max_model_len=MAX_CONTEXT, num_blocks=1 + max_batch * (-(-(PROMPT_LEN + 2 * 1024) // block)),
+              max_num_batched_tokens=max(PREFILL_TOKENS, max_batch), enable_prefix_cache=False)
+    itemsize = 2 if args.dtype == "bf16" else 4
+    wbytes, per_layer_params = weight_bytes(cfg, layers, itemsize)
+    kv_per_token = llm.core.kv_bytes_per_token
+
+    # prefill of 2,048 tokens
+    pre_s = measure_prefill(llm, rng, vocab)
+    h, nq, d = cfg["hidden_size"], cfg["num_attention_heads"], cfg["head_dim"]
+    t = PREFILL_TOKENS
+    flops = 2.0 * t * per_layer_params * layers + 4.0 * nq * d * (t * (t + 1) / 2.0) * layers + 2.0 * vocab * h
+    prefill = {"value": round(t / pre_s, 1), "tokens": t, "ms": round(pre_s * 1e3, 3),
+               "frac": round(flops / pre_s / PEAK_FLOPS[args.dtype], 4)}
+
+    # decode: headline batch, then the other points
+    tps, step_s, mean_ctx = measure_decode(llm, args.batch, args.steps, args.warmup, rng, vocab)
+    read_bytes = wbytes + args.batch * mean_ctx * kv_per_token
+    achieved = read_bytes / step_s / 1e9
+    points = {}
+    if not args.skip_points:
+        for b in (1, 64):
+            n = min(args.steps, 128)
+            points[f"decode_b{b}"] = round(measure_decode(llm, b, n, min(args.warmup, 8), rng, vocab)[0], 1)
+
+    line = {
+        "metric": "decode_tokens_per_s", "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: seeded uniform-random token ids, random-init weights N(0,0.02), norms 1+N(0,0.02)",
+        "config": {
+            "model": "Qwen3-8B-shaped", "layers": layers, "layers_full": QWEN3_8B["num_hidden_layers"],
+            "hidden": cfg["hidden_size"], "q_heads": nq, "kv_heads": cfg["num_key_value_heads"], "head_dim": d,
+            "intermediate": cfg["intermediate_size"], "vocab": vocab, "global_batch": args.batch,
+            "seq_len": PROMPT_LEN, "max_context": MAX_CONTEXT, "mean_decode_context": round(mean_ctx, 1),
+            "page_size": block, "parallelism": "single-gpu", "rope_theta": cfg["rope_theta"],
+            "hip_graphs": bool(llm.config.use_hip_graphs),
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,10 +1,12 @@
 """Device side of the cache: page storage for every run that keeps keys and values, state
 rows for every run that keeps state, and the grouping of runs by need.
 
-Page tensors are ``[pages + 1, kv_heads, page_size, head_dim]`` in the engine's type, zeroed
-once (page 0, the null page, stays zero and is never written).  Layout and zero-init follow
-``jllm/engine/paged.py:26-38`` except that the head axis comes before the slot axis, so one
-head's keys of a page are contiguous for the attention kernels.
+Key pages are ``[pages + 1, kv_heads, page_size, head_dim]``, value pages are stored
+transposed, ``[pages + 1, kv_heads, head_dim, page_size]``, in the engine's type, zeroed once
+(page 0, the null page, stays zero and is never written).  Zero-init follows
+``jllm/engine/paged.py:26-38``; the layout differs: the head axis comes before the slot axis
+so that one head's keys of a page are contiguous, and values are transposed so that the
+matrix-core kernels read 8 consecutive keys of one head element as 16 aligned bytes.
 """
 from __future__ import annotations
 
@@ -38,9 +40,9 @@ def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs:
         if p.cache is not None:
             if p.cache_of is None:
                 g = group_keys.index(p.cache.group_key)
-                shape = (num_pages[g] + 1, p.cache.num_kv_heads, page_size, p.cache.head_dim)
-                mem.k_pages = torch.zeros(shape, dtype=dtype, device=device)
-                mem.v_pages = torch.zeros(shape, dtype=dtype, device=device)
+                n, h, d = num_pages[g] + 1, p.cache.num_kv_heads, p.cache.head_dim
+                mem.k_pages = torch.zeros((n, h, page_size, d), dtype=dtype, device=device)
+                mem.v_pages = torch.zeros((n, h, d, page_size), dtype=dtype, device=device)
                 mem.group, mem.writes = g, True
             else:
                 owner = memories[p.cache_of]

@@ -8,7 +8,7 @@
 //   and sees keys j with  max(0, p - window + 1) <= j <= p   (window <= 0: all j <= p);
 //   key j lives in page block_tables[r, j / page_size] at slot j % page_size;
 //   q head h reads kv head h / (nq / nkv).
-// Cache layout: pages[page][kv_head][slot][D].
+// Cache layout: K pages[page][kv_head][slot][D], V pages[page][kv_head][D][slot].
 #include "common.h"
 
 #define GEN_MAX_E 8  // head size up to 64 * 8
@@ -20,7 +20,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
                                const int* __restrict__ block_tables, int table_stride,
                                const int* __restrict__ token_req, const int* __restrict__ positions,
                                int page_size, int nq, int nkv, int D, float scale, int window) {
-  extern __shared__ float lds[];      // q[D] | p[64] | row offsets as long long [64]
+  extern __shared__ float lds[];      // q[D] | p[64] | V offsets of the tile's keys as long long [64]
   float* qs = lds;
   float* ps = lds + D;
   long long* offs = (long long*)(ps + 64 + ((D & 1) ? 1 : 0));
@@ -48,8 +48,8 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
     long long off = 0;
     if (valid) {
       const long long page = table[j / page_size];
-      off = ((page * nkv + kvh) * page_size + (j % page_size)) * (long long)D;
-      const T* kr = k_pages + off;
+      const T* kr = k_pages + ((page * nkv + kvh) * page_size + (j % page_size)) * (long long)D;
+      off = (page * nkv + kvh) * (long long)D * page_size + (j % page_size);
       float dot = 0.f;
       for (int d = 0; d < D; ++d) dot += qs[d] * to_f32(kr[d]);
       s = dot * scale;
@@ -69,7 +69,7 @@ paged_attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, lon
       const int d = lane + 64 * e;
       if (d < D) {
         float a = acc[e] * alpha;
-        for (int jj = 0; jj < n; ++jj) a += ps[jj] * to_f32(v_pages[offs[jj] + d]);
+        for (int jj = 0; jj < n; ++jj) a += ps[jj] * to_f32(v_pages[offs[jj] + (long long)d * page_size]);
         acc[e] = a;
       }
     }

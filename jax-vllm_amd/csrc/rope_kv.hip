@@ -7,8 +7,10 @@
 // Rotation (float): for pair index p < rotary_dim/2, angle = pos * inv_freq[p];
 //   half-split pairing:  (x[p], x[p + rotary_dim/2])     interleaved: (x[2p], x[2p+1])
 //   (a, b) -> (a*cos - b*sin, b*cos + a*sin);  elements >= rotary_dim pass through.
-// Cache layout: pages[page][kv_head][slot][D]; slot_mapping[t] = page * page_size + slot,
-// or a negative value for a token whose k/v must not be stored.
+// Cache layout: K pages[page][kv_head][slot][D]; V pages[page][kv_head][D][slot] (transposed,
+// so that the attention kernels find a page's keys contiguous per d);
+// slot_mapping[t] = page * page_size + slot, or a negative value for a token whose k/v must
+// not be stored.
 #include "common.h"
 
 #define ROPE_MAX_D 512
@@ -43,8 +45,8 @@ __global__ void qk_norm_rope_write_kernel(
     T* x = row + (long long)(live ? head : 0) * D;
     if (is_v && store) {  // v head: copy to its page
       const int kvh = head - nq - nkv;
-      T* dst = v_pages + ((page * nkv + kvh) * page_size + off) * (long long)D;
-      for (int d = lane; d < D; d += JV_WAVE) dst[d] = x[d];
+      T* dst = v_pages + (page * nkv + kvh) * (long long)D * page_size + off;
+      for (int d = lane; d < D; d += JV_WAVE) dst[(long long)d * page_size] = x[d];
     }
     const bool work = is_q || (is_k && store);  // a k head that nobody will read is skipped
     const float* w = is_q ? q_w : k_w;

@@ -105,6 +105,13 @@ class LLM:
                 events.append(StepEvent(item.request.request_id, int(tok), finished))
         return events
 
+    def abort_all(self) -> None:
+        """Drop every waiting and running request and give back what they hold."""
+        self.scheduler.waiting.clear()
+        for req in list(self.scheduler.running):
+            self.scheduler.finish(req)
+        self.requests.clear()
+
     # ---- blocking use
     def generate(self, prompts: Sequence[Sequence[int]],
                  sampling: Union[SamplingParams, Sequence[SamplingParams], None] = None,

@@ -147,11 +147,21 @@ def silu_mul(gate_up: torch.Tensor, out=None) -> torch.Tensor:
     return out
 
 
+def _check_pages(k_pages, v_pages, dtype, nkv, page_size, head_dim) -> None:
+    _need(k_pages.dtype == dtype and v_pages.dtype == dtype, "cache pages must have the activation type")
+    _need(k_pages.dim() == 4 and tuple(k_pages.shape[1:]) == (nkv, page_size, head_dim),
+          "key pages must be [pages, nkv, page_size, D]")
+    _need(v_pages.dim() == 4 and tuple(v_pages.shape[1:]) == (nkv, head_dim, page_size),
+          "value pages must be [pages, nkv, D, page_size]")
+    _need(k_pages.shape[0] == v_pages.shape[0], "key and value pages differ in number")
+
+
 # --------------------------------------------------------------------------- attention input
 def qk_norm_rope_write(qkv, positions, slot_mapping, q_weight, k_weight, eps, inv_freq, rotary_dim,
                        interleaved, k_pages, v_pages, page_size, nq, nkv, head_dim) -> None:
     """Per-head q/k RMSNorm (if weights given), rotation (if inv_freq given), q in place,
-    k and v into their pages (if pages given).  Cache pages are [pages, nkv, page_size, D]."""
+    k and v into their pages (if pages given): K [pages, nkv, page_size, D], V transposed
+    [pages, nkv, D, page_size]."""
     _dev(qkv, positions, slot_mapping, q_weight, k_weight, inv_freq, k_pages, v_pages)
     n = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.shape[1] == (nq + 2 * nkv) * head_dim, "qkv must be [tokens, (nq + 2 nkv) * D]")
@@ -166,9 +176,7 @@ def qk_norm_rope_write(qkv, positions, slot_mapping, q_weight, k_weight, eps, in
         _f32(inv_freq, "inv_freq", rotary_dim // 2)
     if k_pages is not None:
         _i32(slot_mapping, "slot_mapping", n)
-        for p in (k_pages, v_pages):
-            _need(p.dtype == qkv.dtype and p.dim() == 4 and tuple(p.shape[1:]) == (nkv, page_size, head_dim),
-                  "cache pages must be [pages, nkv, page_size, D] of the activation type")
+        _check_pages(k_pages, v_pages, qkv.dtype, nkv, page_size, head_dim)
     fn = getattr(library.core(), f"jv_qk_norm_rope_write_{_suffix(qkv.dtype)}")
     _check(
         fn(_ptr(qkv), _ptr(positions), _ptr(slot_mapping if k_pages is not None else None), _ptr(q_weight),
@@ -192,9 +200,7 @@ def paged_attention_generic(out, q, q_row_stride, k_pages, v_pages, block_tables
     _need(nkv > 0 and nq % nkv == 0, "q heads must be a multiple of kv heads")
     _need(head_dim <= 512, "head size above 512 is not supported")
     page_size = k_pages.shape[2]
-    for p in (k_pages, v_pages):
-        _need(p.dtype == q.dtype and p.dim() == 4 and tuple(p.shape[1:]) == (nkv, page_size, head_dim),
-              "cache pages must be [pages, nkv, page_size, D] of q's type")
+    _check_pages(k_pages, v_pages, q.dtype, nkv, page_size, head_dim)
     _need(block_tables.dim() == 2, "block_tables must be [requests, pages]")
     _i32(block_tables, "block_tables")
     _i32(token_req, "token_req", n)
@@ -260,3 +266,79 @@ def sample(logits: torch.Tensor, temperature=None, keys=None, out=None) -> torch
     _check(fn(_ptr(out), _ptr(logits), c_longlong(v), c_int(m), c_int(v), _ptr(temperature),
               _ptr(keys if temperature is not None else None), _stream()), "sample")
     return out
+
+
+# --------------------------------------------------------------------------- matrix-core attention (bfloat16)
+MFMA_ATTENTION_MAX_HEAD_DIM = 256
+
+
+def mfma_attention_supported(dtype, head_dim: int, page_size: int) -> bool:
+    """The matrix-core kernels take bfloat16, head sizes that are multiples of 16 up to 256 and
+    page sizes that are multiples of 8; everything else goes to the generic kernel."""
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= MFMA_ATTENTION_MAX_HEAD_DIM
+            and page_size % 8 == 0)
+
+
+def _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, nq, nkv,
+                 head_dim):
+    _dev(out, q, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work)
+    _need(q.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "matrix-core attention takes bfloat16")
+    n = out.shape[0]
+    _need(out.shape == (n, nq * head_dim), "out must be [tokens, nq * D]")
+    _need(q_row_stride % 8 == 0 and q.data_ptr() % 16 == 0, "q rows must be 16-byte aligned")
+    _need(q.numel() >= (n - 1) * q_row_stride + nq * head_dim if n else True, "q is too small for its stride")
+    page_size = k_pages.shape[2]
+    _check_pages(k_pages, v_pages, q.dtype, nkv, page_size, head_dim)
+    _need(page_size % 8 == 0, "page size must be a multiple of 8")
+    _need(block_tables.dim() == 2, "block_tables must be [requests, pages]")
+    for t, name in ((block_tables, "block_tables"), (cu_seqlens, "cu_seqlens"), (context_lens, "context_lens"),
+                    (work, "work")):
+        _i32(t, name)
+    _need(cu_seqlens.numel() == context_lens.numel() + 1 == block_tables.shape[0] + 1,
+          "cu_seqlens, context_lens and block_tables disagree on the number of requests")
+    return page_size
+
+
+def attn_prefill_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, n_work,
+                      nq, nkv, head_dim, scale, window=0) -> None:
+    """Causal attention of prompt portions.  ``work`` is int32 [n_work, 2]: (request index, first row)
+    for every block of 64 rows, a row being a (query, head-in-group) pair of one kv head."""
+    page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
+                             nq, nkv, head_dim)
+    _need(work.numel() >= 2 * n_work, "work list shorter than n_work")
+    lib = library.attention(head_dim)
+    _check(
+        lib.jv_attn_prefill(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages),
+                            _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens),
+                            _ptr(work), c_int(n_work), c_int(page_size), c_int(nq), c_int(nkv), c_float(scale),
+                            c_int(window or 0), _stream()),
+        "attn_prefill_mfma",
+    )
+
+
+def attn_decode_scratch_floats(n_work: int, nq: int, num_splits: int, head_dim: int) -> int:
+    return n_work * nq * num_splits * (head_dim + 2) if num_splits > 1 else 0
+
+
+def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, n_work,
+                     nq, nkv, head_dim, scale, window=0, num_splits=1, scratch=None) -> None:
+    """Attention of single decoded tokens.  ``work`` is int32 [n_work]: indices of the requests
+    (each with exactly one token in this step).  With ``num_splits`` > 1 a request's keys are
+    shared out to that many blocks and ``scratch`` (float32, ``attn_decode_scratch_floats``
+    entries) holds their partial results."""
+    page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
+                             nq, nkv, head_dim)
+    _need(work.numel() >= n_work, "work list shorter than n_work")
+    if num_splits > 1:
+        _need(scratch is not None and scratch.is_cuda and scratch.dtype == torch.float32
+              and scratch.numel() >= attn_decode_scratch_floats(n_work, nq, num_splits, head_dim),
+              "scratch too small for the splits")
+    lib = library.attention(head_dim)
+    _check(
+        lib.jv_attn_decode(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages),
+                           _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens),
+                           _ptr(work), c_int(n_work), c_int(page_size), c_int(nq), c_int(nkv), c_float(scale),
+                           c_int(window or 0), c_int(num_splits), _ptr(scratch if num_splits > 1 else None),
+                           _stream()),
+        "attn_decode_mfma",
+    )

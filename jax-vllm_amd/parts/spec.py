@@ -62,7 +62,8 @@ class StateSpec:
 class LayerMemory:
     """What the cache manager hands one layer run.
 
-    k_pages, v_pages: [pages, kv_heads, page_size, head_dim] or None; ``group`` says which
+    k_pages [pages, kv_heads, page_size, head_dim], v_pages [pages, kv_heads, head_dim,
+    page_size] (transposed), or None; ``group`` says which
     block table / slot mapping of the step applies; ``writes`` is False for a run that reads
     another run's cache.  ``state`` is [slots, *shape] or None.
     """

@@ -136,7 +136,7 @@ def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_nor
     kw = (1 + 0.1 * randn(d, seed=13)) if with_norm else None
     inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))).cuda()
     k_pages = torch.zeros(pages, nkv, page_size, d, dtype=dtype).cuda()
-    v_pages = torch.zeros_like(k_pages)
+    v_pages = torch.zeros(pages, nkv, d, page_size, dtype=dtype).cuda()
     x = qkv.float().view(t, nq + 2 * nkv, d).clone()
     K().qk_norm_rope_write(qkv, pos, slots, qw, kw, eps, inv_freq, rotary_dim, interleaved, k_pages, v_pages,
                            page_size, nq, nkv, d)
@@ -154,11 +154,11 @@ def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_nor
     torch.testing.assert_close(got_q[near.cuda()], q[near.cuda()], **small)
     torch.testing.assert_close(got_q, q, **big)
     exp_k = torch.zeros(pages, nkv, page_size, d).cuda()
-    exp_v = torch.zeros_like(exp_k)
+    exp_v = torch.zeros(pages, nkv, d, page_size).cuda()     # values are stored transposed
     for i, s in enumerate(slots.tolist()):
         if s >= 0:
             exp_k[s // page_size, :, s % page_size] = k[i]
-            exp_v[s // page_size, :, s % page_size] = v[i]
+            exp_v[s // page_size, :, :, s % page_size] = v[i]
     torch.testing.assert_close(k_pages.float(), exp_k, **big)
     torch.testing.assert_close(v_pages.float(), exp_v, rtol=0, atol=0)  # values are copied untouched
     written = torch.zeros(pages * page_size, dtype=torch.bool)
@@ -176,7 +176,7 @@ def build_paged(k, v, page_size, seed=0, extra_pages=3):
     order = (torch.randperm(total - 1, generator=g) + 1).tolist()
     nkv, d = k[0].shape[1], k[0].shape[2]
     k_pages = torch.randn(total, nkv, page_size, d, generator=g) * 50  # garbage where no key lives
-    v_pages = torch.randn(total, nkv, page_size, d, generator=g) * 50
+    v_pages = torch.randn(total, nkv, d, page_size, generator=g) * 50  # values are stored transposed
     tables = torch.zeros(len(k), max(need), dtype=torch.int32)
     for r, (kk, vv) in enumerate(zip(k, v)):
         for p in range(need[r]):
@@ -185,7 +185,7 @@ def build_paged(k, v, page_size, seed=0, extra_pages=3):
             chunk = slice(p * page_size, min((p + 1) * page_size, kk.shape[0]))
             n = chunk.stop - chunk.start
             k_pages[page, :, :n] = kk[chunk].transpose(0, 1)
-            v_pages[page, :, :n] = vv[chunk].transpose(0, 1)
+            v_pages[page, :, :, :n] = vv[chunk].permute(1, 2, 0)
     return k_pages, v_pages, tables
 
 
@@ -301,3 +301,154 @@ def test_temperature_sampling_matches_softmax():
     out3 = K().sample(logits, t2, keys)
     assert (out3[::2] == torch.argmax(logits1[0])).all()
     assert out3[1::2].tolist() == out[1::2].tolist()
+
+
+# ------------------------------------------------------------------ matrix-core attention (bfloat16)
+def _mfma_inputs(nq, nkv, d, page_size, reqs, seed=5):
+    g = torch.Generator().manual_seed(seed)
+    bf = torch.bfloat16
+    ks = [torch.randn(c + q, nkv, d, generator=g).to(bf).float() for c, q in reqs]
+    vs = [torch.randn(c + q, nkv, d, generator=g).to(bf).float() for c, q in reqs]
+    qs = [torch.randn(q, nq, d, generator=g).to(bf).float() for c, q in reqs]
+    k_pages, v_pages, tables = build_paged(ks, vs, page_size, seed=seed)
+    n = sum(q for _, q in reqs)
+    stride = (nq + 2 * nkv) * d
+    qbuf = torch.zeros(n, stride)
+    cu, at = [0], 0
+    for r, (c, ql) in enumerate(reqs):
+        qbuf[at:at + ql, :nq * d] = qs[r].reshape(ql, nq * d)
+        at += ql
+        cu.append(at)
+    dev = dict(
+        q=qbuf.to(bf).cuda(), k_pages=k_pages.to(bf).cuda(), v_pages=v_pages.to(bf).cuda(), tables=tables.cuda(),
+        cu=torch.tensor(cu, dtype=torch.int32).cuda(),
+        ctx=torch.tensor([c for c, _ in reqs], dtype=torch.int32).cuda(), stride=stride, n=n,
+    )
+    return qs, ks, vs, dev
+
+
+def _mfma_reference(qs, ks, vs, reqs, scale, window, nq, d):
+    refs = []
+    for r, (c, ql) in enumerate(reqs):
+        refs.append(attention_reference(qs[r], ks[r], vs[r], torch.arange(c, c + ql), scale, window))
+    return torch.cat(refs).reshape(-1, nq * d)
+
+
+MFMA_PREFILL_CASES = [c for c in ATT_CASES if c[3] % 8 == 0] + [
+    (32, 8, 128, 16, [(0, 200), (1000, 50)], None),
+    (4, 4, 112, 24, [(30, 40), (0, 3)], None),
+    (8, 1, 64, 8, [(5, 70)], 17),
+    (40, 2, 32, 16, [(10, 9)], None),      # 20 heads per group: rows of one query span two 16-row tiles
+]
+
+
+@pytest.mark.parametrize("case", MFMA_PREFILL_CASES,
+                         ids=[f"h{c[0]}g{c[1]}d{c[2]}p{c[3]}w{c[5]}n{len(c[4])}" for c in MFMA_PREFILL_CASES])
+def test_mfma_prefill_attention(case):
+    nq, nkv, d, page_size, reqs, window = case
+    scale = 1.0 / math.sqrt(d)
+    qs, ks, vs, dev = _mfma_inputs(nq, nkv, d, page_size, reqs)
+    g = nq // nkv
+    work = [x for r, (c, ql) in enumerate(reqs) for m0 in range(0, ql * g, 64) for x in (r, m0)]
+    out = torch.full((dev["n"], nq * d), float("nan"), dtype=torch.bfloat16).cuda()
+    K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                          dev["ctx"], torch.tensor(work, dtype=torch.int32).cuda(), len(work) // 2, nq, nkv, d,
+                          scale, window or 0)
+    ref = _mfma_reference(qs, ks, vs, reqs, scale, window, nq, d)
+    torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
+
+
+MFMA_DECODE_CASES = [
+    # nq, nkv, d, page_size, contexts, window
+    (4, 2, 16, 8, [0, 1, 7, 8, 33, 200], None),
+    (6, 2, 32, 16, [9, 100, 31, 32, 1234], None),
+    (5, 5, 48, 32, [37, 0, 500], None),
+    (32, 8, 128, 16, [1023, 1024, 1500, 3], None),
+    (16, 2, 256, 16, [130, 64], None),
+    (40, 2, 64, 16, [77, 300], None),      # 20 heads per group: two row tiles per kv head
+    (8, 2, 64, 16, [50, 200, 1000], 24),
+    (4, 4, 80, 40, [99, 160], None),
+]
+
+
+@pytest.mark.parametrize("splits", [1, 3, 8])
+@pytest.mark.parametrize("case", MFMA_DECODE_CASES,
+                         ids=[f"h{c[0]}g{c[1]}d{c[2]}p{c[3]}w{c[5]}" for c in MFMA_DECODE_CASES])
+def test_mfma_decode_attention(case, splits):
+    nq, nkv, d, page_size, contexts, window = case
+    reqs = [(c, 1) for c in contexts]
+    scale = 1.0 / math.sqrt(d)
+    qs, ks, vs, dev = _mfma_inputs(nq, nkv, d, page_size, reqs, seed=9)
+    # the work list names the requests in another order than they lie in the batch
+    order = list(reversed(range(len(reqs))))
+    scratch = None
+    if splits > 1:
+        scratch = torch.full((K().attn_decode_scratch_floats(len(reqs), nq, splits, d),), float("nan")).cuda()
+    out = torch.full((dev["n"], nq * d), float("nan"), dtype=torch.bfloat16).cuda()
+    K().attn_decode_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                         dev["ctx"], torch.tensor(order, dtype=torch.int32).cuda(), len(order), nq, nkv, d, scale,
+                         window or 0, splits, scratch)
+    ref = _mfma_reference(qs, ks, vs, reqs, scale, window, nq, d)
+    torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
+
+
+@pytest.mark.parametrize("far_key", [0, 15, 16, 31, 32, 63, 64, 255, 256, 511, 640])
+@pytest.mark.parametrize("kernel", ["prefill", "decode1", "decode5"])
+def test_mfma_attention_finds_one_far_key(kernel, far_key):
+    nq, nkv, d, page_size, ctx = 4, 2, 64, 16, 641
+    g = torch.Generator().manual_seed(far_key)
+    k = (torch.randn(ctx, nkv, d, generator=g) * 0.1)
+    v = torch.randn(ctx, nkv, d, generator=g)
+    q = torch.randn(1, nq, d, generator=g) * 0.1
+    q[0, :, 0] = 40.0
+    k[far_key, :, 0] = 40.0
+    bf = torch.bfloat16
+    k_pages, v_pages, tables = build_paged([k.to(bf).float()], [v.to(bf).float()], page_size, seed=far_key)
+    out = torch.empty(1, nq * d, dtype=bf).cuda()
+    args = (out, q.reshape(1, -1).to(bf).cuda(), nq * d, k_pages.to(bf).cuda(), v_pages.to(bf).cuda(), tables.cuda(),
+            torch.tensor([0, 1], dtype=torch.int32).cuda(), torch.tensor([ctx - 1], dtype=torch.int32).cuda())
+    scale = 1.0 / math.sqrt(d)
+    if kernel == "prefill":
+        K().attn_prefill_mfma(*args, torch.tensor([0, 0], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
+    else:
+        splits = int(kernel[-1])
+        scratch = torch.empty(max(1, K().attn_decode_scratch_floats(1, nq, splits, d))).cuda()
+        K().attn_decode_mfma(*args, torch.tensor([0], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale, 0, splits,
+                             scratch)
+    expect = torch.repeat_interleave(v[far_key].to(bf).float(), nq // nkv, dim=0).reshape(1, -1)
+    torch.testing.assert_close(out.float().cpu(), expect, rtol=1e-2, atol=1e-2)
+
+
+def test_mfma_attention_ignores_garbage_past_the_context():
+    """Slots of the last page beyond the context hold NaN and infinity: they must not leak."""
+    nq, nkv, d, page_size = 4, 2, 64, 16
+    reqs = [(0, 21), (37, 1)]
+    qs, ks, vs, dev = _mfma_inputs(nq, nkv, d, page_size, reqs, seed=3)
+    for r, (c, ql) in enumerate(reqs):
+        n = c + ql
+        page = int(dev["tables"][r, n // page_size])
+        dev["k_pages"][page, :, n % page_size:] = float("nan")
+        dev["v_pages"][page, :, :, n % page_size:] = float("inf")
+    scale = 1.0 / math.sqrt(d)
+    ref = _mfma_reference(qs, ks, vs, reqs, scale, None, nq, d)
+    out = torch.zeros(dev["n"], nq * d, dtype=torch.bfloat16).cuda()
+    K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                          dev["ctx"], torch.tensor([0, 0, 0, 64], dtype=torch.int32).cuda(), 2, nq, nkv, d, scale)
+    K().attn_decode_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                         dev["ctx"], torch.tensor([1], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
+    torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
+
+
+def test_mfma_attention_refuses_what_it_cannot_do():
+    from jax_vllm_amd.ops.kernels import KernelArgumentError, mfma_attention_supported
+
+    assert not mfma_attention_supported(torch.bfloat16, 80, 4)       # page size not a multiple of 8
+    assert not mfma_attention_supported(torch.bfloat16, 72, 16)      # head size not a multiple of 16
+    assert not mfma_attention_supported(torch.bfloat16, 272, 16)     # head size above 256
+    assert not mfma_attention_supported(torch.float32, 64, 16)
+    nq, nkv, d, page_size = 3, 1, 80, 4
+    qs, ks, vs, dev = _mfma_inputs(nq, nkv, d, page_size, [(3, 2)])
+    out = torch.zeros(dev["n"], nq * d, dtype=torch.bfloat16).cuda()
+    with pytest.raises(KernelArgumentError, match="multiple of 8"):
+        K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                              dev["ctx"], torch.tensor([0, 0], dtype=torch.int32).cuda(), 1, nq, nkv, d, 0.1)
