@@ -49,6 +49,70 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ 
   }
 }
 
+// The same for widths that are a multiple of 4 and at most 4 * 8 * blockDim: 16-byte loads of
+// the residual stream, the row kept in registers between the two passes.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> { typedef float4 type; };
+template <> struct Vec4<bf16_t> { typedef __attribute__((ext_vector_type(4))) __bf16 type; };
+
+template <typename T>
+__device__ __forceinline__ float4 load4(const T* p) {
+  typename Vec4<T>::type v = *(const typename Vec4<T>::type*)p;
+  return float4{to_f32<T>(v[0]), to_f32<T>(v[1]), to_f32<T>(v[2]), to_f32<T>(v[3])};
+}
+template <>
+__device__ __forceinline__ float4 load4<float>(const float* p) { return *(const float4*)p; }
+
+template <typename T>
+__device__ __forceinline__ void store4(T* p, float4 v) {
+  typename Vec4<T>::type o;
+  o[0] = from_f32<T>(v.x); o[1] = from_f32<T>(v.y); o[2] = from_f32<T>(v.z); o[3] = from_f32<T>(v.w);
+  *(typename Vec4<T>::type*)p = o;
+}
+template <>
+__device__ __forceinline__ void store4<float>(float* p, float4 v) { *(float4*)p = v; }
+
+#define ARN_MAX_V 8
+template <typename T>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                                       const float* __restrict__ w, T* __restrict__ out,
+                                       const int* __restrict__ rows, int hidden, float eps) {
+  __shared__ float red[32];
+  const long long i = blockIdx.x;
+  const long long r = rows ? (long long)rows[i] : i;
+  float* hr = h + r * hidden;
+  const T* dr = delta ? delta + r * hidden : nullptr;
+  T* o = out + i * hidden;
+  const int nvec = hidden >> 2;
+  float4 x[ARN_MAX_V];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < ARN_MAX_V; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c < nvec) {
+      float4 v = *(const float4*)(hr + 4 * c);
+      if (dr) {
+        const float4 d = load4<T>(dr + 4 * c);
+        v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+        if (!rows) *(float4*)(hr + 4 * c) = v;
+      }
+      x[k] = v;
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+  for (int k = 0; k < ARN_MAX_V; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c < nvec) {
+      const float4 ww = *(const float4*)(w + 4 * c);
+      const float4 v = x[k];
+      store4<T>(o + 4 * c, float4{v.x * inv * ww.x, v.y * inv * ww.y, v.z * inv * ww.z, v.w * inv * ww.w});
+    }
+  }
+}
+
 // ---------------------------------------------------------------- plain RMSNorm over the last axis
 // out[r, :] = T( x[r,:] * rsqrt(mean(x^2)+eps) * w ), x of type T, rows of length n.
 // One wave per row, several rows per block.
@@ -72,16 +136,21 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* __restrict__ x,
 
 // ---------------------------------------------------------------- SiLU-mul
 // out[t, j] = silu(gu[t, j]) * gu[t, inter + j], silu(x) = x / (1 + exp(-x)), in float.
-template <typename T>
-__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, long long total,
-                                int inter) {
-  const long long stride = (long long)gridDim.x * blockDim.x;
-  for (long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += stride) {
-    const long long t = e / inter;
-    const int j = (int)(e - t * inter);
-    const float g = to_f32(gu[t * 2 * inter + j]);
-    const float u = to_f32(gu[t * 2 * inter + inter + j]);
-    out[e] = from_f32<T>(g / (1.f + expf(-g)) * u);
+// grid (column blocks, tokens); each thread takes 4 neighbouring columns when inter % 4 == 0.
+template <typename T, int VEC>
+__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
+  const long long t = blockIdx.y;
+  const int j = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+  if (j >= inter) return;
+  const T* gp = gu + t * 2 * inter + j;
+  T* op = out + t * inter + j;
+  if (VEC == 4) {
+    const float4 g = load4<T>(gp), u = load4<T>(gp + inter);
+    store4<T>(op, float4{g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
+                         g.z / (1.f + expf(-g.z)) * u.z, g.w / (1.f + expf(-g.w)) * u.w});
+  } else {
+    const float g = to_f32(gp[0]), u = to_f32(gp[inter]);
+    op[0] = from_f32<T>(g / (1.f + expf(-g)) * u);
   }
 }
 
@@ -107,8 +176,15 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
                                       void* stream) {                                               \
     if (n_out <= 0) return 0;                                                                       \
     const int threads = hidden >= 2048 ? 512 : 256;                                                 \
-    hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(threads), 0, (hipStream_t)stream,   \
-                       h, (const T*)delta, w, (T*)out, rows, hidden, eps);                          \
+    if (hidden % 4 == 0 && hidden <= 4 * ARN_MAX_V * 256) {                                         \
+      const int nvec = hidden / 4;                                                                  \
+      const int vt = nvec >= 1024 ? 256 : (nvec >= 256 ? 128 : 64);                                 \
+      hipLaunchKernelGGL(add_rmsnorm_vec_kernel<T>, dim3(n_out), dim3(vt), 0, (hipStream_t)stream,  \
+                         h, (const T*)delta, w, (T*)out, rows, hidden, eps);                        \
+    } else {                                                                                        \
+      hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(threads), 0, (hipStream_t)stream, \
+                         h, (const T*)delta, w, (T*)out, rows, hidden, eps);                        \
+    }                                                                                               \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \
   extern "C" int jv_rmsnorm_##SUF(void* out, const void* x, const float* w, long long rows, int n,  \
@@ -122,12 +198,19 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
   }                                                                                                 \
   extern "C" int jv_silu_mul_##SUF(void* out, const void* gu, long long n_tokens, int inter,        \
                                    void* stream) {                                                  \
-    const long long total = n_tokens * inter;                                                       \
-    if (total <= 0) return 0;                                                                       \
-    long long blocks = (total + 255) / 256;                                                         \
-    if (blocks > 65536) blocks = 65536;                                                             \
-    hipLaunchKernelGGL(silu_mul_kernel<T>, dim3((unsigned)blocks), dim3(256), 0,                    \
-                       (hipStream_t)stream, (T*)out, (const T*)gu, total, inter);                   \
+    if (n_tokens <= 0 || inter <= 0) return 0;                                                      \
+    for (long long t0 = 0; t0 < n_tokens; t0 += 65535) { /* grid.y limit */                         \
+      const unsigned ny = (unsigned)(n_tokens - t0 < 65535 ? n_tokens - t0 : 65535);                \
+      T* o = (T*)out + t0 * inter;                                                                  \
+      const T* g = (const T*)gu + t0 * 2 * inter;                                                   \
+      if (inter % 4 == 0) {                                                                         \
+        hipLaunchKernelGGL((silu_mul_kernel<T, 4>), dim3((inter / 4 + 255) / 256, ny), dim3(256),   \
+                           0, (hipStream_t)stream, o, g, inter);                                    \
+      } else {                                                                                      \
+        hipLaunchKernelGGL((silu_mul_kernel<T, 1>), dim3((inter + 255) / 256, ny), dim3(256), 0,    \
+                           (hipStream_t)stream, o, g, inter);                                       \
+      }                                                                                             \
+    }                                                                                               \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \
   extern "C" int jv_cast_rows_##SUF(void* out, const float* x, const int* rows, int n_out, int n,   \

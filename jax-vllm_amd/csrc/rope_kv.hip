@@ -4,7 +4,8 @@
 // Input is the fused projection output qkv[t, (nq + 2*nkv) * D]; head j of q is
 // columns [j*D, (j+1)*D), then the k heads, then the v heads.
 //
-// Rotation (float): for pair index p < rotary_dim/2, angle = pos * inv_freq[p];
+// Rotation (float): for pair index p < rotary_dim/2, angle = pos * inv_freq[p], cosine and sine
+// taken from a per-step table;
 //   half-split pairing:  (x[p], x[p + rotary_dim/2])     interleaved: (x[2p], x[2p+1])
 //   (a, b) -> (a*cos - b*sin, b*cos + a*sin);  elements >= rotary_dim pass through.
 // Cache layout: K pages[page][kv_head][slot][D]; V pages[page][kv_head][D][slot] (transposed,
@@ -15,90 +16,105 @@
 
 #define ROPE_MAX_D 512
 
+// cos_sin[t, 0:half] = cos(pos_t * inv_freq), cos_sin[t, half:2*half] = sin(...), all float.
+// Computed once per step: every layer of the step rotates by the same angles.
+__global__ void rope_table_kernel(float* __restrict__ cos_sin, const int* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, int half) {
+  const long long t = blockIdx.x;
+  const float pos = (float)positions[t];
+  for (int p = threadIdx.x; p < half; p += blockDim.x) {
+    float s, c;
+    sincosf(pos * inv_freq[p], &s, &c);
+    cos_sin[t * 2 * half + p] = c;
+    cos_sin[t * 2 * half + half + p] = s;
+  }
+}
+
+extern "C" int jv_rope_table(float* cos_sin, const int* positions, const float* inv_freq,
+                             int n_tokens, int half, void* stream) {
+  if (n_tokens <= 0 || half <= 0) return 0;
+  hipLaunchKernelGGL(rope_table_kernel, dim3(n_tokens), dim3(half >= 128 ? 128 : 64), 0,
+                     (hipStream_t)stream, cos_sin, positions, inv_freq, half);
+  return JV_LAUNCH_CHECK();
+}
+
+// One wave per (token, head); 4 heads per block.
 template <typename T>
-__global__ void qk_norm_rope_write_kernel(
-    T* __restrict__ qkv, const int* __restrict__ positions, const int* __restrict__ slot_mapping,
-    const float* __restrict__ q_w, const float* __restrict__ k_w, float eps,
-    const float* __restrict__ inv_freq, int rotary_dim, int interleaved, T* __restrict__ k_pages,
-    T* __restrict__ v_pages, int page_size, int nq, int nkv, int D) {
-  extern __shared__ float lds[];  // [waves][D]
+__global__ void __launch_bounds__(256) qk_norm_rope_write_kernel(
+    T* __restrict__ qkv, const int* __restrict__ slot_mapping, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, float eps, const float* __restrict__ cos_sin, int rotary_dim,
+    int interleaved, T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size, int nq,
+    int nkv, int D) {
+  extern __shared__ float lds[];  // [4 waves][D]
   const int lane = threadIdx.x & (JV_WAVE - 1), wid = threadIdx.x / JV_WAVE;
-  const int nwaves = blockDim.x / JV_WAVE;
   float* buf = lds + wid * D;
   const long long t = blockIdx.x;
   const int n_heads = nq + 2 * nkv;
+  const int head = blockIdx.y * 4 + wid;
+  const bool live = head < n_heads;
   T* row = qkv + t * (long long)n_heads * D;
-  const float pos = (float)positions[t];
   const long long slot = slot_mapping ? (long long)slot_mapping[t] : -1;
   const bool store = (slot >= 0) && (k_pages != nullptr);
   const long long page = store ? slot / page_size : 0;
   const int off = store ? (int)(slot - page * page_size) : 0;
   const int half = rotary_dim / 2;
-
-  // Every wave runs the same number of rounds so that the block barriers line up.
-  for (int base = 0; base < n_heads; base += nwaves) {
-    const int head = base + wid;
-    const bool live = head < n_heads;
-    const bool is_v = live && head >= nq + nkv;
-    const bool is_q = live && head < nq;
-    const bool is_k = live && !is_q && !is_v;
-    T* x = row + (long long)(live ? head : 0) * D;
-    if (is_v && store) {  // v head: copy to its page
-      const int kvh = head - nq - nkv;
-      T* dst = v_pages + (page * nkv + kvh) * (long long)D * page_size + off;
-      for (int d = lane; d < D; d += JV_WAVE) dst[(long long)d * page_size] = x[d];
+  const bool is_v = live && head >= nq + nkv;
+  const bool is_q = live && head < nq;
+  const bool is_k = live && !is_q && !is_v;
+  T* x = row + (long long)(live ? head : 0) * D;
+  if (is_v && store) {  // v head: copied to its (transposed) page
+    const int kvh = head - nq - nkv;
+    T* dst = v_pages + (page * nkv + kvh) * (long long)D * page_size + off;
+    for (int d = lane; d < D; d += JV_WAVE) dst[(long long)d * page_size] = x[d];
+  }
+  const bool work = is_q || (is_k && store);  // a k head that nobody will read is skipped
+  const float* w = is_q ? q_w : k_w;
+  if (work) {
+    float ss = 0.f;
+    for (int d = lane; d < D; d += JV_WAVE) {
+      const float v = to_f32(x[d]);
+      buf[d] = v;
+      ss += v * v;
     }
-    const bool work = is_q || (is_k && store);  // a k head that nobody will read is skipped
-    const float* w = is_q ? q_w : k_w;
-    if (work) {
-      float ss = 0.f;
-      for (int d = lane; d < D; d += JV_WAVE) {
-        const float v = to_f32(x[d]);
-        buf[d] = v;
-        ss += v * v;
-      }
-      if (w) {
-        ss = wave_sum(ss);
-        const float inv = rsqrtf(ss / (float)D + eps);
-        for (int d = lane; d < D; d += JV_WAVE) buf[d] = buf[d] * inv * w[d];
-      }
+    if (w) {
+      ss = wave_sum(ss);
+      const float inv = rsqrtf(ss / (float)D + eps);
+      for (int d = lane; d < D; d += JV_WAVE) buf[d] = buf[d] * inv * w[d];
     }
-    __syncthreads();  // buf written -> readable by the wave's other lanes
-    if (work) {
-      T* dst = is_q ? x
-                    : k_pages + ((page * nkv + (head - nq)) * page_size + off) * (long long)D;
-      if (inv_freq) {
-        for (int p = lane; p < half; p += JV_WAVE) {
-          const int ia = interleaved ? 2 * p : p;
-          const int ib = interleaved ? 2 * p + 1 : p + half;
-          float s, c;
-          sincosf(pos * inv_freq[p], &s, &c);
-          const float a = buf[ia], b = buf[ib];
-          dst[ia] = from_f32<T>(a * c - b * s);
-          dst[ib] = from_f32<T>(b * c + a * s);
-        }
-        for (int d = rotary_dim + lane; d < D; d += JV_WAVE) dst[d] = from_f32<T>(buf[d]);
-      } else {
-        for (int d = lane; d < D; d += JV_WAVE) dst[d] = from_f32<T>(buf[d]);
+  }
+  __syncthreads();  // buf written -> readable by the wave's other lanes (every wave arrives once)
+  if (work) {
+    T* dst = is_q ? x : k_pages + ((page * nkv + (head - nq)) * page_size + off) * (long long)D;
+    if (cos_sin) {
+      const float* cs = cos_sin + t * rotary_dim;
+      for (int p = lane; p < half; p += JV_WAVE) {
+        const int ia = interleaved ? 2 * p : p;
+        const int ib = interleaved ? 2 * p + 1 : p + half;
+        const float c = cs[p], sn = cs[half + p];
+        const float a = buf[ia], b = buf[ib];
+        dst[ia] = from_f32<T>(a * c - b * sn);
+        dst[ib] = from_f32<T>(b * c + a * sn);
       }
+      for (int d = rotary_dim + lane; d < D; d += JV_WAVE) dst[d] = from_f32<T>(buf[d]);
+    } else {
+      for (int d = lane; d < D; d += JV_WAVE) dst[d] = from_f32<T>(buf[d]);
     }
-    __syncthreads();  // buf is reused in the next round
   }
 }
 
 #define DEFINE_ROPE(SUF, T)                                                                        \
   extern "C" int jv_qk_norm_rope_write_##SUF(                                                      \
-      void* qkv, const int* positions, const int* slot_mapping, const float* q_w,                  \
-      const float* k_w, float eps, const float* inv_freq, int rotary_dim, int interleaved,         \
-      void* k_pages, void* v_pages, int page_size, int n_tokens, int nq, int nkv, int D,           \
-      void* stream) {                                                                              \
+      void* qkv, const int* slot_mapping, const float* q_w, const float* k_w, float eps,           \
+      const float* cos_sin, int rotary_dim, int interleaved, void* k_pages, void* v_pages,         \
+      int page_size, int n_tokens, int nq, int nkv, int D, void* stream) {                         \
     if (n_tokens <= 0) return 0;                                                                   \
     if (D > ROPE_MAX_D || rotary_dim > D || (rotary_dim & 1)) return (int)hipErrorInvalidValue;    \
-    const int waves = 4;                                                                           \
-    hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(n_tokens), dim3(waves * JV_WAVE),        \
-                       waves * D * sizeof(float), (hipStream_t)stream, (T*)qkv, positions,         \
-                       slot_mapping, q_w, k_w, eps, inv_freq, rotary_dim, interleaved,             \
-                       (T*)k_pages, (T*)v_pages, page_size, nq, nkv, D);                           \
+    const int n_heads = nq + 2 * nkv;                                                              \
+    if ((n_heads + 3) / 4 > 65535) return (int)hipErrorInvalidValue;                               \
+    hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(n_tokens, (n_heads + 3) / 4), dim3(256), \
+                       4 * D * sizeof(float), (hipStream_t)stream, (T*)qkv, slot_mapping, q_w,     \
+                       k_w, eps, cos_sin, rotary_dim, interleaved, (T*)k_pages, (T*)v_pages,       \
+                       page_size, nq, nkv, D);                                                     \
     return JV_LAUNCH_CHECK();                                                                      \
   }
 

@@ -27,6 +27,55 @@ from ..parts.spec import StepContext
 from ..weights.loader import TORCH_DTYPES
 
 
+def _bucket(n: int, floor: int = 1) -> int:
+    """The next power of two at or above n (and at least ``floor``)."""
+    b = floor
+    while b < n:
+        b *= 2
+    return b
+
+
+class _DecodeGraph:
+    """Fixed host and device buffers of one captured decode step and the graph itself."""
+
+    def __init__(self, rb: int, widths: tuple, n_groups: int, device):
+        names = [("tokens", rb), ("positions", rb), ("token_req", rb), ("cu", rb + 1), ("ctx", rb), ("slots", rb),
+                 ("rows", rb)]
+        names += [(f"slot_mapping{g}", rb) for g in range(n_groups)]
+        names += [(f"table{g}", rb * widths[g]) for g in range(n_groups)]
+        self.rb, self.widths, self.n_groups = rb, widths, n_groups
+        self.offsets, at = {}, 0
+        for name, size in names:
+            self.offsets[name] = (at, at + size)
+            at += size
+        self.host_tensor = torch.zeros(at, dtype=torch.int32, pin_memory=True)
+        self.host = self.host_tensor.numpy()
+        self.dev = torch.zeros(at, dtype=torch.int32, device=device)
+        self.graph = None
+        self.logits = None
+        self.ctx = None
+
+    def segment(self, host, name):
+        a, b = self.offsets[name]
+        return host[a:b]
+
+    def dev_segment(self, name):
+        a, b = self.offsets[name]
+        return self.dev[a:b]
+
+    def context(self, page_size: int, max_kv_len: int) -> StepContext:
+        rb = self.rb
+        return StepContext(
+            num_tokens=rb, num_requests=rb, positions=self.dev_segment("positions"),
+            token_req=self.dev_segment("token_req"), cu_seqlens=self.dev_segment("cu"),
+            context_lens=self.dev_segment("ctx"), slot_ids=self.dev_segment("slots"),
+            block_tables=[self.dev_segment(f"table{g}").view(rb, self.widths[g]) for g in range(self.n_groups)],
+            slot_mappings=[self.dev_segment(f"slot_mapping{g}") for g in range(self.n_groups)],
+            page_size=page_size, q_lens_host=[1] * rb, context_lens_host=[max_kv_len - 1] * rb,
+            slot_ids_host=[0] * rb, max_q_len=1, max_kv_len=max_kv_len,
+        )
+
+
 @dataclass
 class StepEntry:
     """One request's share of a step: its next tokens and the indices among them (0-based)
@@ -55,6 +104,9 @@ class EngineCore:
                                           config.max_num_seqs, self.dtype, self.device)
         self.vocab_size = model.spec.vocab_size
         self.kv_bytes_per_token = cache_bytes_per_token(self.plan, self.dtype)
+        self._graphs: dict = {}
+        self._max_graph_batch = min(config.max_num_seqs, 256)
+        self.graph_replays = 0
 
     # ---- requests
     def start_request(self, request_id, prompt: Optional[Sequence[int]] = None) -> int:
@@ -68,9 +120,11 @@ class EngineCore:
         return self.cache.has(request_id)
 
     # ---- the step
-    def run(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def run(self, entries: Sequence[StepEntry], borrow: bool = False) -> torch.Tensor:
         """Float logits [wanted, vocab] in the order of the entries and of their ``want``.
-        Raises ``OutOfPages`` before anything ran if a request's tokens have no room."""
+        Raises ``OutOfPages`` before anything ran if a request's tokens have no room.
+        ``borrow``: the caller reads the logits before the next call, so a replayed step may
+        hand out its own output buffer instead of a copy."""
         entries = [e for e in entries if len(e.tokens) > 0]
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.device)
@@ -83,12 +137,74 @@ class EngineCore:
                     raise ValueError(f"request {e.request_id!r}: wanted place {w} outside its {len(e.tokens)} tokens")
         for e in entries:
             self.cache.reserve(e.request_id, len(e.tokens))
-        token_ids, ctx, logit_rows = self._build(entries)
         self._zero_new_state()
-        logits = self.model.forward(token_ids, ctx, self.memories, logit_rows)
+        if self._graphable(entries):
+            logits = self._run_decode_graph(entries)
+            if not borrow:
+                logits = logits.clone()
+        else:
+            token_ids, ctx, logit_rows = self._build(entries)
+            logits = self.model.forward(token_ids, ctx, self.memories, logit_rows)
         for e in entries:
             self.cache.commit(e.request_id, e.tokens)
         return logits
+
+    # ---- decode-only steps as replayed HIP graphs
+    def _graphable(self, entries) -> bool:
+        if not self.config.use_hip_graphs or len(entries) > self._max_graph_batch:
+            return False
+        return all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
+
+    def _run_decode_graph(self, entries) -> torch.Tensor:
+        """A step of single tokens, one per request, each wanting its logits: the launch sequence
+        is captured once per (batch bucket, table-width bucket) and replayed from fixed buffers;
+        rows added to reach the bucket size read the null page and store nothing."""
+        cache, ps = self.cache, self.page_size
+        r = len(entries)
+        rb = _bucket(r)
+        n_groups = len(self.group_keys)
+        tables = [[cache.block_table(e.request_id, g) for e in entries] for g in range(n_groups)]
+        widths = tuple(_bucket(max(len(t) for t in tables[g]), 8) for g in range(n_groups))
+        key = (rb, widths)
+        g = self._graphs.get(key)
+        if g is None:
+            g = self._graphs[key] = _DecodeGraph(rb, widths, n_groups, self.device)
+        host = g.host
+        host[:] = 0
+        seg = g.segment
+        ctx_lens = [cache.context_len(e.request_id) for e in entries]
+        seg(host, "tokens")[:r] = [int(e.tokens[0]) for e in entries]
+        seg(host, "positions")[:r] = ctx_lens
+        seg(host, "token_req")[:] = np.arange(rb, dtype=np.int32)
+        seg(host, "cu")[:] = np.arange(rb + 1, dtype=np.int32)
+        seg(host, "ctx")[:r] = ctx_lens
+        seg(host, "slots")[:r] = [cache.slot(e.request_id) for e in entries]
+        seg(host, "rows")[:] = np.arange(rb, dtype=np.int32)
+        for gi in range(n_groups):
+            sm = seg(host, f"slot_mapping{gi}")
+            sm[:] = -1
+            sm[:r] = [cache.slot_mapping(e.request_id, gi, 1)[0] for e in entries]
+            bt = seg(host, f"table{gi}").reshape(rb, widths[gi])
+            for i, t in enumerate(tables[gi]):
+                bt[i, :len(t)] = t
+        g.dev.copy_(g.host_tensor, non_blocking=True)
+        if g.graph is None:
+            # first use: run the launches eagerly (this is the step's result), then record them
+            ctx = g.context(ps, self.page_size * max(widths, default=1))
+            logits = self.model.forward(g.dev_segment("tokens"), ctx, self.memories, g.dev_segment("rows"))
+            g.logits = torch.empty_like(logits)
+            g.logits.copy_(logits)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            ctx.extras = {}   # per-step kernel results are recomputed inside the graph; plans stay
+            with torch.cuda.graph(graph):
+                out = self.model.forward(g.dev_segment("tokens"), ctx, self.memories, g.dev_segment("rows"))
+                g.logits.copy_(out)
+            g.graph, g.ctx = graph, ctx
+        else:
+            g.graph.replay()
+            self.graph_replays += 1
+        return g.logits[:r]
 
     def _zero_new_state(self) -> None:
         slots = self.cache.take_new_slots()

@@ -85,7 +85,7 @@ class LLM:
                 self.stats.prefill_portions += 1
         self.stats.steps_run += 1
         self.stats.max_batched_tokens = max(self.stats.max_batched_tokens, out.num_tokens)
-        logits = self.core.run(entries)
+        logits = self.core.run(entries, borrow=True)
         temps = [i.request.sampling.temperature for i in sampled]
         keys = [
             draw_key(i.request.sampling.seed if i.request.sampling.seed is not None else self.config.seed,

@@ -157,30 +157,43 @@ def _check_pages(k_pages, v_pages, dtype, nkv, page_size, head_dim) -> None:
 
 
 # --------------------------------------------------------------------------- attention input
-def qk_norm_rope_write(qkv, positions, slot_mapping, q_weight, k_weight, eps, inv_freq, rotary_dim,
-                       interleaved, k_pages, v_pages, page_size, nq, nkv, head_dim) -> None:
-    """Per-head q/k RMSNorm (if weights given), rotation (if inv_freq given), q in place,
-    k and v into their pages (if pages given): K [pages, nkv, page_size, D], V transposed
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out=None) -> torch.Tensor:
+    """float32 [tokens, 2 * half]: cos(pos * inv_freq) then sin(pos * inv_freq), angles in float."""
+    _dev(positions, inv_freq, out)
+    n, half = positions.numel(), inv_freq.numel()
+    _i32(positions, "positions")
+    _f32(inv_freq, "inv_freq")
+    if out is None:
+        out = torch.empty((n, 2 * half), dtype=torch.float32, device=positions.device)
+    _need(out.shape == (n, 2 * half) and out.dtype == torch.float32, "table must be float32 [tokens, 2 * half]")
+    _check(library.core().jv_rope_table(_ptr(out), _ptr(positions), _ptr(inv_freq), c_int(n), c_int(half),
+                                        _stream()), "rope_table")
+    return out
+
+
+def qk_norm_rope_write(qkv, slot_mapping, q_weight, k_weight, eps, cos_sin, rotary_dim, interleaved,
+                       k_pages, v_pages, page_size, nq, nkv, head_dim) -> None:
+    """Per-head q/k RMSNorm (if weights given), rotation (if a ``rope_table`` is given), q in
+    place, k and v into their pages (if pages given): K [pages, nkv, page_size, D], V transposed
     [pages, nkv, D, page_size]."""
-    _dev(qkv, positions, slot_mapping, q_weight, k_weight, inv_freq, k_pages, v_pages)
+    _dev(qkv, slot_mapping, q_weight, k_weight, cos_sin, k_pages, v_pages)
     n = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.shape[1] == (nq + 2 * nkv) * head_dim, "qkv must be [tokens, (nq + 2 nkv) * D]")
-    _i32(positions, "positions", n)
     _need(head_dim <= 512, "head size above 512 is not supported by the rotation kernel")
     if q_weight is not None:
         _f32(q_weight, "q_weight", head_dim)
     if k_weight is not None:
         _f32(k_weight, "k_weight", head_dim)
-    if inv_freq is not None:
+    if cos_sin is not None:
         _need(rotary_dim % 2 == 0 and 0 < rotary_dim <= head_dim, "rotary_dim must be even and at most D")
-        _f32(inv_freq, "inv_freq", rotary_dim // 2)
+        _f32(cos_sin, "cos_sin", n * rotary_dim)
     if k_pages is not None:
         _i32(slot_mapping, "slot_mapping", n)
         _check_pages(k_pages, v_pages, qkv.dtype, nkv, page_size, head_dim)
     fn = getattr(library.core(), f"jv_qk_norm_rope_write_{_suffix(qkv.dtype)}")
     _check(
-        fn(_ptr(qkv), _ptr(positions), _ptr(slot_mapping if k_pages is not None else None), _ptr(q_weight),
-           _ptr(k_weight), c_float(eps), _ptr(inv_freq), c_int(rotary_dim if inv_freq is not None else 0),
+        fn(_ptr(qkv), _ptr(slot_mapping if k_pages is not None else None), _ptr(q_weight), _ptr(k_weight),
+           c_float(eps), _ptr(cos_sin), c_int(rotary_dim if cos_sin is not None else 0),
            c_int(1 if interleaved else 0), _ptr(k_pages), _ptr(v_pages), c_int(page_size), c_int(n),
            c_int(nq), c_int(nkv), c_int(head_dim), _stream()),
         "qk_norm_rope_write",

@@ -65,13 +65,13 @@ class GroupedQueryAttention:
     def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
         n = x.shape[0]
         qkv = K.linear(x, self.w_qkv)
-        inv_freq, rotary_dim, interleaved = (
-            self.position.fused_arguments() if self.position is not None else (None, 0, False)
+        cos_sin, rotary_dim, interleaved = (
+            self.position.fused_arguments(ctx) if self.position is not None else (None, 0, False)
         )
         writes = mem.writes
         K.qk_norm_rope_write(
-            qkv, ctx.positions, ctx.slot_mappings[mem.group] if writes else None, self.q_norm, self.k_norm,
-            self.qk_norm_eps or 0.0, inv_freq, rotary_dim, interleaved,
+            qkv, ctx.slot_mappings[mem.group] if writes else None, self.q_norm, self.k_norm,
+            self.qk_norm_eps or 0.0, cos_sin, rotary_dim, interleaved,
             mem.k_pages if writes else None, mem.v_pages if writes else None, ctx.page_size,
             self.nq, self.nkv, self.d,
         )

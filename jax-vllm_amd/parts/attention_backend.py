@@ -72,9 +72,9 @@ def run(att, out, qkv, ctx, mem) -> None:
         )
         return
     key = ("mfma_attention_plan", att.nq, att.nkv, att.d)
-    plan = ctx.extras.get(key)
+    plan = ctx.plans.get(key)
     if plan is None:
-        plan = ctx.extras[key] = plan_mfma(ctx, att.nq, att.nkv, att.d, qkv.device)
+        plan = ctx.plans[key] = plan_mfma(ctx, att.nq, att.nkv, att.d, qkv.device)
     tables = ctx.block_tables[mem.group]
     if plan.n_prefill:
         K.attn_prefill_mfma(out, qkv, q_row_stride, mem.k_pages, mem.v_pages, tables, ctx.cu_seqlens,

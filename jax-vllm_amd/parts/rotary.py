@@ -4,13 +4,15 @@
 float; the pair (i, i + dim/2) of a head vector (half-split pairing, the reference's
 ``_rotate_half``) turns by its angle.  ``rotary_dim`` (default: the whole head) and
 ``interleaved`` pairing (2i, 2i+1) are parameters; elements past ``rotary_dim`` pass
-through.  The rotation itself runs inside the attention-input kernel, which takes
-this part's table and flags; cos and sin stay in float there.
+through.  Cosines and sines of a step's positions are computed once per step, in float,
+and shared by every layer with the same constants; the rotation itself runs inside the
+attention-input kernel, which takes that table and this part's flags.
 """
 from __future__ import annotations
 
 import torch
 
+from ..ops import kernels as K
 from .spec import register_part
 
 
@@ -35,9 +37,14 @@ class RotaryEncoding:
     def bind(self, tensors: dict, dtype: torch.dtype, device=None) -> None:
         self.inv_freq = self.inverse_frequencies().to(device or "cuda").contiguous()
 
-    def fused_arguments(self):
-        """(inv_freq, rotary_dim, interleaved) for the attention-input kernel."""
-        return self.inv_freq, self.rotary_dim, self.interleaved
+    def fused_arguments(self, ctx):
+        """(cos/sin table of the step's positions, rotary_dim, interleaved) for the
+        attention-input kernel."""
+        key = ("rope_table", self.theta, self.rotary_dim)
+        table = ctx.extras.get(key)
+        if table is None:
+            table = ctx.extras[key] = K.rope_table(ctx.positions, self.inv_freq)
+        return table, self.rotary_dim, self.interleaved
 
 
 register_part("position", "rotary", RotaryEncoding)

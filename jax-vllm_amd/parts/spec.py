@@ -98,7 +98,8 @@ class StepContext:
     slot_ids_host: list                # [R]
     max_q_len: int = 1
     max_kv_len: int = 1
-    extras: dict = field(default_factory=dict)   # per-step scratch shared by parts of one kind
+    extras: dict = field(default_factory=dict)   # per-step results of kernels, shared by parts of one kind
+    plans: dict = field(default_factory=dict)    # per-step work lists built on the host and uploaded
 
     @property
     def decode_only(self) -> bool:

@@ -138,7 +138,10 @@ def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_nor
     k_pages = torch.zeros(pages, nkv, page_size, d, dtype=dtype).cuda()
     v_pages = torch.zeros(pages, nkv, d, page_size, dtype=dtype).cuda()
     x = qkv.float().view(t, nq + 2 * nkv, d).clone()
-    K().qk_norm_rope_write(qkv, pos, slots, qw, kw, eps, inv_freq, rotary_dim, interleaved, k_pages, v_pages,
+    table = K().rope_table(pos, inv_freq)
+    ang = pos.float()[:, None] * inv_freq[None, :]
+    torch.testing.assert_close(table, torch.cat([torch.cos(ang), torch.sin(ang)], dim=1), rtol=1e-5, atol=2e-6)
+    K().qk_norm_rope_write(qkv, slots, qw, kw, eps, table, rotary_dim, interleaved, k_pages, v_pages,
                            page_size, nq, nkv, d)
     q, k, v = x[:, :nq], x[:, nq:nq + nkv], x[:, nq + nkv:]
     if with_norm:
