@@ -1,0 +1,231 @@
+// y[M,N] = x[M,K] * W[N,K]^T for few rows (M <= 64), bf16 in, float accumulate: the
+// weight-streaming matrix product of decode steps, bound by HBM bandwidth.
+//
+// v_mfma_f32_16x16x32_bf16 with A = 16 rows of W, B = 16 rows of x (both K-contiguous, so
+// every lane loads 16 contiguous bytes per operand and nothing is transposed); the
+// accumulator holds y^T[n][m].
+//
+// A block has WR x WK waves: wave (wr, wk) owns W rows [16*(WR*block + wr), +16) and, of
+// every K chunk of WK*STEP columns, the slice wk.  W goes from global memory straight into
+// MFMA operands, one step ahead of its use.  x must not take that road (it would double
+// the vector-memory traffic of a kernel that lives on it): the block copies only the valid
+// rows of each x chunk into LDS once, double-buffered, and all its waves read their B
+// operands from there.  Partial tiles of the WK slices are added through LDS in a fixed
+// order, so a result does not depend on M, on the grid or on timing.
+//
+// Optional prologue for the feed-forward's second product: x = silu(gate) * up computed
+// (in float) from gate_up[M, 2K] while the chunk is copied into LDS, which saves the
+// activation kernel and its round trip.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define SK_PAD 8  // bf16 elements of padding per LDS row (keeps 16-byte reads of 16 rows off the same banks)
+
+template <int MT, int NKS, typename OutT, bool SILU>
+__global__ void __launch_bounds__(1024)
+gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
+                   int M, int N, int K, long long ldx, long long ldy, int WR, int WK) {
+  constexpr int STEP = NKS * 32;
+  constexpr int ROWS = MT * 16;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  const int KCB = WK * STEP;                 // columns of one x chunk
+  const int LROW = KCB + SK_PAD;             // LDS row length in elements
+  bf16_t* xs = (bf16_t*)smem;                // [2][ROWS][LROW]
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int wave = tid >> 6, lane = tid & 63, li = lane & 15, lc = lane >> 4;
+  const int wr = wave % WR, wk = wave / WR;
+  const int n = (blockIdx.x * WR + wr) * 16 + li;
+  const bool n_ok = n < N;
+  const bf16_t* wrow = W + (long long)(n_ok ? n : 0) * K + lc * 8;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int n_iter = (K + KCB - 1) / KCB;
+
+  // rows M..ROWS-1 of both buffers stay zero for the whole kernel
+  for (int c = tid; c < 2 * ROWS * LROW / 8; c += nthreads) *(bf16x8*)(xs + c * 8) = zero;
+  __syncthreads();
+
+  // chunk `it` of x (valid rows only) -> registers -> LDS buffer
+  const int xvecs = M * (KCB / 8);           // 16-byte pieces of one chunk
+  auto load_x_piece = [&](int it, int c) -> bf16x8 {
+    const int m = c / (KCB / 8), kc = c - m * (KCB / 8);
+    const int k = it * KCB + kc * 8;
+    if (k >= K) return zero;
+    if (!SILU) return *(const bf16x8*)(x + (long long)m * ldx + k);
+    const bf16_t* g = x + (long long)m * ldx + k;
+    const bf16x8 gv = *(const bf16x8*)g, uv = *(const bf16x8*)(g + K);
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gf = (float)gv[e], uf = (float)uv[e];
+      r[e] = (bf16_t)(gf / (1.f + expf(-gf)) * uf);
+    }
+    return r;
+  };
+  auto store_x_piece = [&](int buf, int c, bf16x8 v) {
+    const int m = c / (KCB / 8), kc = c - m * (KCB / 8);
+    *(bf16x8*)(xs + (buf * ROWS + m) * LROW + kc * 8) = v;
+  };
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 a_cur[NKS], a_nxt[NKS];
+  auto load_w = [&](int it, bf16x8* a) {
+    const int k0 = it * KCB + wk * STEP;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const int k = k0 + ks * 32 + lc * 8;
+      a[ks] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k0 + ks * 32) : zero;
+    }
+  };
+  // prologue: chunk 0 into buffer 0, W of iteration 0
+  for (int c = tid; c < xvecs; c += nthreads) store_x_piece(0, c, load_x_piece(0, c));
+  load_w(0, a_cur);
+
+  for (int it = 0; it < n_iter; ++it) {
+    const bool more = it + 1 < n_iter;
+    if (more) load_w(it + 1, a_nxt);
+    // next chunk's pieces of this thread: at most 2 in flight in registers, the rest (large M
+    // with few threads) are copied after the products
+    bf16x8 xr0 = zero, xr1 = zero;
+    const int c0 = tid, c1 = tid + nthreads;
+    if (more) {
+      if (c0 < xvecs) xr0 = load_x_piece(it + 1, c0);
+      if (c1 < xvecs) xr1 = load_x_piece(it + 1, c1);
+    }
+    __syncthreads();  // buffer it&1 is complete; everyone is done reading buffer (it+1)&1
+    const bf16_t* xb = xs + ((it & 1) * ROWS) * LROW + wk * STEP + lc * 8;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 b = *(const bf16x8*)(xb + (mt * 16 + li) * LROW + ks * 32);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[ks], b, acc[mt], 0, 0, 0);
+      }
+    }
+    if (more) {
+      const int nb = (it + 1) & 1;
+      if (c0 < xvecs) store_x_piece(nb, c0, xr0);
+      if (c1 < xvecs) store_x_piece(nb, c1, xr1);
+      for (int c = tid + 2 * nthreads; c < xvecs; c += nthreads) store_x_piece(nb, c, load_x_piece(it + 1, c));
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) a_cur[ks] = a_nxt[ks];
+    }
+  }
+
+  // ---- fixed-order sum over the WK slices; tile of wave (wr, wk), row tile mt, at
+  //      red[((wk * WR + wr) * MT + mt) * 256 + lane * 4]
+  __syncthreads();  // the x buffers are free now and are reused for the reduction
+  float* red = (float*)smem;
+  if (WK > 1) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *(f32x4*)(red + (((wk * WR + wr) * MT + mt) * 256 + lane * 4)) = acc[mt];
+    __syncthreads();
+  }
+  // the WK waves of one row tile share its MT column tiles out between them
+  for (int mt = wk; mt < MT; mt += WK) {
+    f32x4 s = WK > 1 ? *(const f32x4*)(red + ((wr * MT + mt) * 256 + lane * 4)) : acc[mt];
+    for (int w = 1; w < WK; ++w) {
+      const f32x4 t = *(const f32x4*)(red + (((w * WR + wr) * MT + mt) * 256 + lane * 4));
+      s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
+    }
+    const int m = mt * 16 + li;
+    const int nb = (blockIdx.x * WR + wr) * 16 + lc * 4;
+    if (m < M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (nb + e < N) y[(long long)m * ldy + nb + e] = from_f32<OutT>(s[e]);
+    }
+  }
+}
+
+static size_t skinny_shmem(int MT, int NKS, int WR, int WK) {
+  const size_t xbytes = (size_t)2 * MT * 16 * (WK * NKS * 32 + SK_PAD) * 2;
+  const size_t rbytes = WK > 1 ? (size_t)WR * WK * MT * 256 * 4 : 0;
+  return xbytes > rbytes ? xbytes : rbytes;
+}
+
+template <int MT, int NKS, typename OutT, bool SILU>
+static int launch_skinny(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
+                         long long ldy, int WR, int WK, hipStream_t stream) {
+  const size_t shmem = skinny_shmem(MT, NKS, WR, WK);
+  if (shmem > 64 * 1024) {
+    static bool raised = false;  // per instantiation
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NKS, OutT, SILU>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return (int)e;
+      raised = true;
+    }
+  }
+  const int blocks = (N + 16 * WR - 1) / (16 * WR);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NKS, OutT, SILU>), dim3(blocks), dim3(WR * WK * 64), shmem,
+                     stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, WR, WK);
+  return JV_LAUNCH_CHECK();
+}
+
+template <int NKS, typename OutT, bool SILU>
+static int dispatch_mt(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
+                       long long ldy, int WR, int WK, hipStream_t s) {
+  switch ((M + 15) / 16) {
+    case 1: return launch_skinny<1, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 2: return launch_skinny<2, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 3: return launch_skinny<3, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 4: return launch_skinny<4, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+template <typename OutT, bool SILU>
+static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, int N, int K,
+                        long long ldx, long long ldy, int WR, int WK, hipStream_t s) {
+  switch (nks) {
+    case 2: return dispatch_mt<2, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 4: return dispatch_mt<4, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 8: return dispatch_mt<8, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+  }
+  return (int)hipErrorInvalidValue;
+}
+
+// Shape of the block chosen from the problem.  Measured on MI355X (weights beyond the last-level
+// cache): one row tile per block with 8 K slices of 128 columns streams fastest for up to 16
+// rows of x at every matrix shape of an 8B-class model; more row tiles per block lose more to
+// the wider barrier than they save on x.
+static void skinny_config(int M, int N, int K, int* wr, int* wk, int* nks) {
+  const int MT = (M + 15) / 16;
+  int WR = 1, WK = 8, NKS = 4;
+  // LDS: 2 * MT*16 rows * WK*NKS*32 columns * 2 bytes <= 64 KB  ->  MT * WK * NKS <= 32
+  while (MT * WK * NKS > 32 && NKS > 2) NKS /= 2;
+  while (MT * WK * NKS > 32 && WK > 1) WK /= 2;
+  // at least two iterations per wave, or the prefetch has nothing to hide
+  while (WK > 1 && K < 2 * WK * NKS * 32) WK /= 2;
+  while (NKS > 2 && K < 2 * WK * NKS * 32) NKS /= 2;
+  (void)N;
+  *wr = WR; *wk = WK; *nks = NKS;
+}
+
+// out_f32: 0 -> y is bf16, 1 -> y is float.  silu: 0 -> x is [M, K] with row stride ldx;
+// 1 -> x is gate_up [M, 2K] (row stride ldx), the product runs on silu(gate) * up, y is bf16.
+// wr, wk, nks: block shape (row tiles, K slices, MFMA steps per iteration); 0 picks them.
+extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
+                                   long long ldx, long long ldy, int out_f32, int silu, int wr,
+                                   int wk, int nks, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
+  if (silu && out_f32) return (int)hipErrorInvalidValue;
+  int cwr, cwk, cnks;
+  skinny_config(M, N, K, &cwr, &cwk, &cnks);
+  if (wr <= 0) wr = cwr;
+  if (wk <= 0) wk = cwk;
+  if (nks <= 0) nks = cnks;
+  const int MT = (M + 15) / 16;
+  if (wr * wk > 16 || (nks != 2 && nks != 4 && nks != 8)) return (int)hipErrorInvalidValue;
+  if (skinny_shmem(MT, nks, wr, wk) > 160 * 1024) return (int)hipErrorInvalidValue;
+  hipStream_t s = (hipStream_t)stream;
+  if (silu) return dispatch_nks<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
+  if (out_f32) return dispatch_nks<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
+  return dispatch_nks<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
+}

@@ -1,4 +1,5 @@
-// Token choice from float logits [M, V], one block per row.
+// Token choice from float logits [M, V] in two stages: many blocks per row each find the winner
+// of a slice of the vocabulary, then one small block per row picks among them.
 //   temperature[r] <= 0 : greedy, the lowest index among the maxima;
 //   temperature[r] >  0 : a draw from softmax(logits / temperature) by the Gumbel-max
 //     rule: argmax_i( logits[i] / T + g_i ), g_i = -log(-log(u_i)), where u_i in (0,1)
@@ -19,48 +20,95 @@ __device__ __forceinline__ float uniform_open01(uint64_t key, uint32_t i) {
   return ((float)(bits >> 40) + 0.5f) * (1.0f / 16777216.0f);
 }
 
-__global__ void __launch_bounds__(256)
-sample_kernel(int* __restrict__ out, const float* __restrict__ logits, long long row_stride, int V,
-              const float* __restrict__ temperature, const unsigned long long* __restrict__ keys) {
+struct Best { float v; int i; };
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) { return v > bv || (v == bv && i < bi); }
+
+// Reduces (value, index) over the block; thread 0 returns the winner.
+__device__ __forceinline__ Best block_best(float best, int best_i) {
   __shared__ float bv[4];
   __shared__ int bi[4];
-  const long long r = blockIdx.x;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best, o, 64);
+    const int oi = __shfl_xor(best_i, o, 64);
+    if (better(ov, oi, best, best_i)) { best = ov; best_i = oi; }
+  }
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  if (lane == 0) { bv[wid] = best; bi[wid] = best_i; }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+      if (better(bv[w], bi[w], best, best_i)) { best = bv[w]; best_i = bi[w]; }
+  return Best{best, best_i};
+}
+
+// Stage 1: grid (chunks, rows); block (c, r) scans columns [c * chunk, (c+1) * chunk) of row r and
+// writes its winner to part[r, c].  Stage 2: grid (rows); reduces the chunks' winners.
+__global__ void __launch_bounds__(256)
+sample_stage1_kernel(float* __restrict__ part_v, int* __restrict__ part_i, const float* __restrict__ logits,
+                     long long row_stride, int V, int chunk, const float* __restrict__ temperature,
+                     const unsigned long long* __restrict__ keys) {
+  const long long r = blockIdx.y;
+  const int c = blockIdx.x;
   const float* row = logits + r * row_stride;
   const float temp = temperature ? temperature[r] : 0.f;
   const uint64_t key = keys ? keys[r] : 0ull;
   const float inv_t = temp > 0.f ? 1.f / temp : 1.f;
   float best = -INFINITY;
   int best_i = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += blockDim.x) {
+  const int end = (c + 1) * chunk < V ? (c + 1) * chunk : V;
+  for (int i = c * chunk + threadIdx.x; i < end; i += blockDim.x) {
     float v = row[i] * inv_t;
-    if (temp > 0.f) {
-      const float u = uniform_open01(key, (uint32_t)i);
-      v += -logf(-logf(u));
-    }
-    if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+    if (temp > 0.f) v += -logf(-logf(uniform_open01(key, (uint32_t)i)));
+    if (better(v, i, best, best_i)) { best = v; best_i = i; }
   }
-  // NaN logits never win a comparison; a row of them yields index 0x7fffffff -> reported as V
+  const Best b = block_best(best, best_i);
+  if (threadIdx.x == 0) {
+    part_v[r * gridDim.x + c] = b.v;
+    part_i[r * gridDim.x + c] = b.i;
+  }
+}
+
+__global__ void __launch_bounds__(64)
+sample_stage2_kernel(int* __restrict__ out, const float* __restrict__ part_v, const int* __restrict__ part_i,
+                     int chunks, int V) {
+  const long long r = blockIdx.x;
+  float best = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += 64) {
+    const float v = part_v[r * chunks + c];
+    const int i = part_i[r * chunks + c];
+    if (better(v, i, best, best_i)) { best = v; best_i = i; }
+  }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     const float ov = __shfl_xor(best, o, 64);
     const int oi = __shfl_xor(best_i, o, 64);
-    if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    if (better(ov, oi, best, best_i)) { best = ov; best_i = oi; }
   }
-  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
-  if (lane == 0) { bv[wid] = best; bi[wid] = best_i; }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
-      if (bv[w] > best || (bv[w] == best && bi[w] < best_i)) { best = bv[w]; best_i = bi[w]; }
-    out[r] = best_i < V ? best_i : V;
-  }
+  // NaN logits never win a comparison; a row of them is reported as V
+  if (threadIdx.x == 0) out[r] = best_i < V ? best_i : V;
 }
 
+#define SAMPLE_MAX_CHUNKS 64
+
+// scratch: SAMPLE_MAX_CHUNKS * n_rows floats followed by as many ints (jv_sample_scratch_bytes)
+extern "C" long long jv_sample_scratch_bytes(int n_rows) { return (long long)n_rows * SAMPLE_MAX_CHUNKS * 8; }
+
 extern "C" int jv_sample(int* out, const float* logits, long long row_stride, int n_rows, int V,
-                         const float* temperature, const unsigned long long* keys, void* stream) {
+                         const float* temperature, const unsigned long long* keys, void* scratch,
+                         void* stream) {
   if (n_rows <= 0) return 0;
-  if (V <= 0) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(256), 0, (hipStream_t)stream, out, logits,
-                     row_stride, V, temperature, keys);
+  if (V <= 0 || !scratch || n_rows > 65535) return (int)hipErrorInvalidValue;
+  int chunks = (V + 4095) / 4096;  // at least 4096 columns per block
+  if (chunks > SAMPLE_MAX_CHUNKS) chunks = SAMPLE_MAX_CHUNKS;
+  const int chunk = (V + chunks - 1) / chunks;
+  float* pv = (float*)scratch;
+  int* pi = (int*)(pv + (long long)n_rows * SAMPLE_MAX_CHUNKS);
+  hipLaunchKernelGGL(sample_stage1_kernel, dim3(chunks, n_rows), dim3(256), 0, (hipStream_t)stream, pv, pi,
+                     logits, row_stride, V, chunk, temperature, keys);
+  int e = JV_LAUNCH_CHECK();
+  if (e) return e;
+  hipLaunchKernelGGL(sample_stage2_kernel, dim3(n_rows), dim3(64), 0, (hipStream_t)stream, out, pv, pi, chunks, V);
   return JV_LAUNCH_CHECK();
 }

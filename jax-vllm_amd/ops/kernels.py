@@ -246,16 +246,57 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out=None) -> torch.Tensor:
     return out
 
 
+SKINNY_MAX_ROWS = 64
+SKINNY_AUTO_ROWS = 16   # up to here ``linear`` prefers the streaming kernel to the library
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_gate_up: bool = False,
+                block_shape=(0, 0, 0), out=None) -> torch.Tensor:
+    """x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w [N, K]: the weight-streaming
+    product of decode steps.  With ``silu_gate_up`` x is gate_up [M, 2K] and the product runs on
+    silu(gate) * up (bfloat16 output only).  Output bfloat16 or float32.  ``block_shape``:
+    (row tiles, K slices, MFMA steps per iteration) of a block, zeros: chosen from the shape."""
+    _dev(x, w, out)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
+    m = x.shape[0]
+    n, k = w.shape
+    _need(x.dim() == 2 and x.shape[1] == (2 * k if silu_gate_up else k), "inner sizes differ")
+    _need(m <= SKINNY_MAX_ROWS, f"gemm_skinny takes at most {SKINNY_MAX_ROWS} rows")
+    _need(k % 8 == 0, "the inner size must be a multiple of 8")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
+    _need(not (silu_gate_up and out_dtype != torch.bfloat16), "the silu prologue writes bfloat16 only")
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    _need(out.shape == (m, n) and out.dtype == out_dtype, "out must be [M, N] of the output type")
+    _check(
+        library.core().jv_gemm_skinny_bf16(
+            _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.shape[1]), c_longlong(n),
+            c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_gate_up else 0),
+            c_int(block_shape[0]), c_int(block_shape[1]), c_int(block_shape[2]), _stream()),
+        "gemm_skinny",
+    )
+    return out
+
+
+def skinny_applies(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``linear`` would run the streaming kernel for these operands."""
+    return x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[0] <= SKINNY_AUTO_ROWS \
+        and w.shape[1] % 8 == 0
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:
     """x @ w.T for w stored [out, in].
 
     float32: the library's own float-FMA kernel (no reduced-precision matrix mode).
-    bfloat16: a plain library matrix product (hipBLASLt through torch), float accumulation.
+    bfloat16, at most 64 rows: the weight-streaming MFMA kernel of this library.
+    bfloat16, more rows: a plain library matrix product (hipBLASLt through torch), float accumulation.
     """
     if x.dtype == torch.float32:
         y = gemm_f32(x, w)
     else:
         _need(x.dtype == w.dtype, "x and w must have one type")
+        if skinny_applies(x, w):
+            return gemm_skinny(x, w, out_dtype or torch.bfloat16)
         y = torch.mm(x, w.t())
     if out_dtype is not None and y.dtype != out_dtype:
         y = y.to(out_dtype)
@@ -275,9 +316,11 @@ def sample(logits: torch.Tensor, temperature=None, keys=None, out=None) -> torch
         _need(keys is not None and keys.dtype == torch.int64 and keys.numel() == m, "keys must be int64, one per row")
     if out is None:
         out = torch.empty((m,), dtype=torch.int32, device=logits.device)
-    fn = library.core().jv_sample
-    _check(fn(_ptr(out), _ptr(logits), c_longlong(v), c_int(m), c_int(v), _ptr(temperature),
-              _ptr(keys if temperature is not None else None), _stream()), "sample")
+    lib = library.core()
+    lib.jv_sample_scratch_bytes.restype = c_longlong
+    scratch = torch.empty(lib.jv_sample_scratch_bytes(c_int(m)), dtype=torch.uint8, device=logits.device)
+    _check(lib.jv_sample(_ptr(out), _ptr(logits), c_longlong(v), c_int(m), c_int(v), _ptr(temperature),
+                         _ptr(keys if temperature is not None else None), _ptr(scratch), _stream()), "sample")
     return out
 
 
@@ -355,3 +398,17 @@ def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_se
                            _stream()),
         "attn_decode_mfma",
     )
+
+
+# --------------------------------------------------------------------------- cache warming
+_prefetch_sink = {}
+
+
+def prefetch(t: torch.Tensor, blocks: int = 64) -> None:
+    """Reads a tensor's bytes with a few workgroups so that they sit in the memory-side cache."""
+    _dev(t)
+    sink = _prefetch_sink.get(t.device)
+    if sink is None:
+        sink = _prefetch_sink[t.device] = torch.zeros(1, dtype=torch.float32, device=t.device)
+    _check(library.core().jv_prefetch(_ptr(t), c_longlong(t.numel() * t.element_size()), c_int(blocks), _ptr(sink),
+                                      _stream()), "prefetch")

@@ -30,6 +30,10 @@ class GatedMLP:
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         gate_up = K.linear(x, self.w_gate_up)
+        if gate_up.shape[0] <= 2 and K.skinny_applies(gate_up, self.w_down):
+            # one or two rows: the activation runs inside the second product's prologue (every
+            # block of that product redoes it, which costs more than a kernel beyond two rows)
+            return K.gemm_skinny(gate_up, self.w_down, gate_up.dtype, silu_gate_up=True)
         return K.linear(K.silu_mul(gate_up), self.w_down)
 
 

@@ -455,3 +455,37 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     with pytest.raises(KernelArgumentError, match="multiple of 8"):
         K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
                               dev["ctx"], torch.tensor([0, 0], dtype=torch.int32).cuda(), 1, nq, nkv, d, 0.1)
+
+
+# ------------------------------------------------------------------ weight-streaming matrix product
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("m,n,k,shape", [
+    (1, 96, 64, (0, 0, 0)), (8, 224, 96, (0, 0, 0)), (33, 520, 136, (2, 3, 2)), (64, 100, 4096, (0, 0, 0)),
+    (5, 777, 80, (1, 16, 2)), (17, 64, 12288, (1, 8, 4)), (3, 30, 264, (1, 1, 8)), (16, 48, 2056, (0, 0, 0)),
+    (8, 24576, 512, (0, 0, 0)), (48, 6144, 1024, (4, 4, 2)), (1, 6144, 4096, (1, 8, 4)), (9, 160, 4096, (4, 4, 8))])
+def test_gemm_skinny(m, n, k, shape, out_dtype):
+    x = randn(m, k, dtype=torch.bfloat16, seed=30, scale=0.5)
+    w = randn(n, k, dtype=torch.bfloat16, seed=31, scale=0.5)
+    out = K().gemm_skinny(x, w, out_dtype, block_shape=shape)
+    ref = x.double() @ w.double().T
+    if out_dtype == torch.float32:
+        # float accumulation of exact bf16 products
+        torch.testing.assert_close(out.double(), ref, rtol=1e-4, atol=1e-4 * math.sqrt(k))
+    else:
+        torch.testing.assert_close(out.double(), ref, rtol=1e-2, atol=1e-2 * math.sqrt(k) / 4)
+    # a row's result does not depend on the other rows of the batch: bit for bit with a fixed
+    # block shape (fixed summation order), to rounding when the shape is chosen from M
+    if m > 1:
+        one = K().gemm_skinny(x[2:3].contiguous() if m > 2 else x[:1].contiguous(), w, out_dtype, block_shape=shape)
+        exact = dict(rtol=0, atol=0) if shape != (0, 0, 0) else dict(rtol=1e-2, atol=1e-3)
+        torch.testing.assert_close(one, out[2:3] if m > 2 else out[:1], **exact)
+
+
+@pytest.mark.parametrize("m,inter,n", [(1, 176, 80), (8, 12288, 96), (40, 224, 100)])
+def test_gemm_skinny_silu_prologue(m, inter, n):
+    gu = randn(m, 2 * inter, dtype=torch.bfloat16, seed=32, scale=2.0)
+    w = randn(n, inter, dtype=torch.bfloat16, seed=33, scale=0.3)
+    out = K().gemm_skinny(gu, w, torch.bfloat16, silu_gate_up=True)
+    z = (torch.nn.functional.silu(gu.float()[:, :inter]) * gu.float()[:, inter:]).to(torch.bfloat16)
+    ref = z.double() @ w.double().T
+    torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=2e-2 * math.sqrt(inter) / 4)
