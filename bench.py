@@ -73,7 +73,7 @@ def measure_decode(llm, batch, steps, warmup, rng, vocab):
 
 
 def measure_prefill(llm, rng, vocab, repeats=3):
-    from jax_vllm_amd.engine.core import StepEntry
+    from jax_vllm_amd.engine.entries import StepEntry
 
     core = llm.core
     best = None

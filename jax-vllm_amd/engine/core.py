@@ -22,6 +22,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.storage import allocate_memories, cache_bytes_per_token, group_keys_of, has_state
 from ..config.engine import EngineConfig
+from .entries import StepEntry
 from ..parts.model import DecoderModel
 from ..parts.spec import StepContext
 from ..weights.loader import TORCH_DTYPES
@@ -74,16 +75,6 @@ class _DecodeGraph:
             page_size=page_size, q_lens_host=[1] * rb, context_lens_host=[max_kv_len - 1] * rb,
             slot_ids_host=[0] * rb, max_q_len=1, max_kv_len=max_kv_len,
         )
-
-
-@dataclass
-class StepEntry:
-    """One request's share of a step: its next tokens and the indices among them (0-based)
-    whose logits are wanted."""
-
-    request_id: object
-    tokens: Sequence[int]
-    want: Sequence[int] = field(default_factory=list)
 
 
 class EngineCore:

@@ -10,37 +10,24 @@ from pathlib import Path
 from typing import Mapping, Optional, Sequence, Union
 
 from ..config.engine import EngineConfig
-from ..sampling.sampler import Sampler, draw_key
-from .core import EngineCore, StepEntry
+from ..sampling.keys import draw_key
+from .entries import StepEntry
 from .request import EngineStats, Request, SamplingParams, StepEvent
 from .scheduler import Scheduler
 
 
-class LLM:
-    """One model on one GPU behind a continuous-batching scheduler.
+class Engine:
+    """The host loop above the step function: requests in, ``StepEvent``s out.  It needs a cache
+    manager for the scheduler, a ``run(entries, borrow=True)`` that returns logits for the
+    wanted places, and a ``sample(logits, temperatures, keys)``; the GPU engine passes the real
+    ones, host-only tests pass stand-ins."""
 
-    ``model`` is a model folder (``config.json`` + safetensors), or a ``config.json``-style
-    dict for random weights drawn on the device from ``random_seed``, or an already bound
-    ``DecoderModel``.  The other arguments are the fields of ``EngineConfig``; the reference's
-    names (``max_num_seqs``, ``max_model_len``, ``max_prefill_len``, ``block_size``,
-    ``num_blocks``, ``dtype`` = "bf16" | "fp32") keep their meaning.
-    """
-
-    def __init__(self, model, *, random_seed: int = 0, device="cuda", **engine_options):
-        from ..parts.model import DecoderModel
-        from ..weights import load_model, random_model_on_device
-
-        self.config = EngineConfig(**engine_options)
-        if isinstance(model, DecoderModel):
-            self.model = model
-        elif isinstance(model, Mapping):
-            self.model, self.model_config = random_model_on_device(model, random_seed, self.config.dtype, device=device)
-        else:
-            self.model, self.model_config = load_model(Path(model), self.config.dtype, device)
-        self.core = EngineCore(self.model, self.config)
+    def __init__(self, config: EngineConfig, cache, run, sample, vocab_size: int):
+        self.config = config
         self.stats = EngineStats()
-        self.scheduler = Scheduler(self.config, self.core.cache, self.stats)
-        self.sampler = Sampler(self.core.device)
+        self.scheduler = Scheduler(config, cache, self.stats)
+        self._run, self._sample = run, sample
+        self.vocab_size = vocab_size
         self._next_id = 0
         self.requests: dict = {}
 
@@ -48,10 +35,9 @@ class LLM:
     def add_request(self, prompt_ids: Sequence[int], sampling: Optional[SamplingParams] = None,
                     arrival_step: int = 0) -> int:
         sp = sampling or SamplingParams()
-        vocab = self.core.vocab_size
         for t in prompt_ids:
-            if not 0 <= int(t) < vocab:
-                raise ValueError(f"token id {t} outside the vocabulary [0, {vocab})")
+            if not 0 <= int(t) < self.vocab_size:
+                raise ValueError(f"token id {t} outside the vocabulary [0, {self.vocab_size})")
         if sp.max_new_tokens < 1:
             raise ValueError("max_new_tokens must be at least 1")
         rid = self._next_id
@@ -85,14 +71,14 @@ class LLM:
                 self.stats.prefill_portions += 1
         self.stats.steps_run += 1
         self.stats.max_batched_tokens = max(self.stats.max_batched_tokens, out.num_tokens)
-        logits = self.core.run(entries, borrow=True)
+        logits = self._run(entries, borrow=True)
         temps = [i.request.sampling.temperature for i in sampled]
         keys = [
             draw_key(i.request.sampling.seed if i.request.sampling.seed is not None else self.config.seed,
                      i.request.request_id, len(i.request.output_ids))
             for i in sampled
         ]
-        tokens = self.sampler.sample(logits, temps, keys)
+        tokens = self._sample(logits, temps, keys)
         events, k = [], 0
         for item in out.items:
             tok = None
@@ -127,6 +113,34 @@ class LLM:
         for r in rids:
             del self.requests[r]
         return outs
+
+
+class LLM(Engine):
+    """One model on one GPU behind a continuous-batching scheduler.
+
+    ``model`` is a model folder (``config.json`` + safetensors), or a ``config.json``-style
+    dict for random weights drawn on the device from ``random_seed``, or an already bound
+    ``DecoderModel``.  The other arguments are the fields of ``EngineConfig``; the reference's
+    names (``max_num_seqs``, ``max_model_len``, ``max_prefill_len``, ``block_size``,
+    ``num_blocks``, ``dtype`` = "bf16" | "fp32") keep their meaning.
+    """
+
+    def __init__(self, model, *, random_seed: int = 0, device="cuda", **engine_options):
+        from ..parts.model import DecoderModel
+        from ..sampling.sampler import Sampler
+        from ..weights import load_model, random_model_on_device
+        from .core import EngineCore
+
+        config = EngineConfig(**engine_options)
+        if isinstance(model, DecoderModel):
+            self.model = model
+        elif isinstance(model, Mapping):
+            self.model, self.model_config = random_model_on_device(model, random_seed, config.dtype, device=device)
+        else:
+            self.model, self.model_config = load_model(Path(model), config.dtype, device)
+        self.core = EngineCore(self.model, config)
+        self.sampler = Sampler(self.core.device)
+        super().__init__(config, self.core.cache, self.core.run, self.sampler.sample, self.core.vocab_size)
 
 
 # ---- the reference's functional spelling ------------------------------------------------

@@ -53,7 +53,8 @@ def main(argv=None, stdin=None, stdout=None) -> int:
     from ..config.engine import EngineConfig
     from ..ops import library
     from ..weights import load_model
-    from .core import EngineCore, StepEntry
+    from .core import EngineCore
+    from .entries import StepEntry
 
     if not torch.cuda.is_available():
         _say("no GPU visible: the engine has no CPU path")

@@ -8,19 +8,12 @@ so it is the same under any batching, cutting or recomputation.
 """
 from __future__ import annotations
 
-import hashlib
 from typing import Sequence
 
 import torch
 
 from ..ops import kernels as K
-
-
-def draw_key(seed: int, request_key: int, index: int) -> int:
-    """64-bit key (as a signed int64 value) of one draw."""
-    d = hashlib.blake2b(f"{seed}:{request_key}:{index}".encode(), digest_size=8).digest()
-    v = int.from_bytes(d, "little")
-    return v - (1 << 64) if v >= (1 << 63) else v
+from .keys import draw_key  # noqa: F401  (re-exported)
 
 
 class Sampler:

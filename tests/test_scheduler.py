@@ -1,0 +1,246 @@
+"""The scheduler's decisions, on the host alone: the real cache manager and the real loop,
+with a stand-in for the step function whose "model" is a fixed function of a request's whole
+token sequence, so that the expected output does not depend on how the work was cut."""
+import hashlib
+
+import numpy as np
+import pytest
+
+from jax_vllm_amd.cache import CacheManager
+from jax_vllm_amd.config import EngineConfig
+from jax_vllm_amd.engine.llm import Engine
+from jax_vllm_amd.engine.request import SamplingParams
+
+VOCAB = 97
+
+
+def next_token(seq) -> int:
+    return int.from_bytes(hashlib.sha256(repr(list(seq)).encode()).digest()[:4], "little") % VOCAB
+
+
+def expected(prompt, n, eos=None):
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = next_token(seq)
+        out.append(t)
+        seq.append(t)
+        if eos is not None and t == eos:
+            break
+    return out
+
+
+class FakeCore:
+    """Does to the cache manager what the step function does, and logs every step."""
+
+    def __init__(self, cfg, groups=(("full",),)):
+        self.cache = CacheManager(list(groups), cfg.page_size, cfg.usable_pages, cfg.max_num_seqs,
+                                  cfg.enable_prefix_cache)
+        self.steps = []
+
+    def run(self, entries, borrow=False):
+        for e in entries:
+            self.cache.reserve(e.request_id, len(e.tokens))
+        rows, log = [], []
+        for e in entries:
+            ctx = self.cache.requests[e.request_id].tokens
+            log.append((e.request_id, len(ctx), len(e.tokens), list(e.want)))
+            rows += [next_token(ctx + list(e.tokens[:w + 1])) for w in e.want]
+        for e in entries:
+            self.cache.commit(e.request_id, e.tokens)
+        self.cache.check_invariants()
+        self.steps.append(log)
+        return rows
+
+    @staticmethod
+    def sample(rows, temps, keys):
+        assert len(rows) == len(temps) == len(keys)
+        return rows
+
+
+def make(**kw):
+    cfg = EngineConfig(**kw)
+    core = FakeCore(cfg)
+    return Engine(cfg, core.cache, core.run, core.sample, VOCAB), core
+
+
+def drain(eng, limit=5000):
+    events = []
+    while eng.has_work():
+        events.append(eng.step())
+        limit -= 1
+        assert limit > 0, "the engine does not finish"
+    return events
+
+
+def test_two_requests_share_one_step_and_budget_is_respected():
+    eng, core = make(block_size=4, max_num_seqs=4, max_model_len=64, max_num_batched_tokens=16)
+    a = eng.add_request(list(range(10)), SamplingParams(max_new_tokens=3))
+    b = eng.add_request(list(range(20, 29)), SamplingParams(max_new_tokens=3))
+    drain(eng)
+    # step 0: a whole (10 tokens) and the first 6 of b under the budget of 16; step 1: a decodes
+    # first (one token), then b's remaining 3 tokens
+    assert core.steps[0] == [(a, 0, 10, [9]), (b, 0, 6, [])]
+    assert core.steps[1] == [(a, 10, 1, [0]), (b, 6, 3, [2])]
+    assert all(sum(n for _, _, n, _ in s) <= 16 for s in core.steps)
+    assert eng.stats.max_batched_tokens == 16 and eng.stats.admissions == 2
+    assert eng.stats.emitted_tokens == 6 and eng.stats.decode_tokens == 4 and eng.stats.prefill_tokens == 19
+
+
+def test_outputs_do_not_depend_on_budget_chunk_or_pages():
+    rng = np.random.default_rng(0)
+    prompts = [rng.integers(0, VOCAB, size=n).tolist() for n in (1, 9, 40, 64, 100)]
+    want = [expected(p, 12) for p in prompts]
+    for kw in (dict(max_num_batched_tokens=2048), dict(max_num_batched_tokens=24), dict(max_num_batched_tokens=7, max_chunk=3),
+               dict(max_num_batched_tokens=24, num_blocks=1 + 12), dict(max_num_batched_tokens=5, num_blocks=1 + 8, max_num_seqs=2)):
+        eng, core = make(**dict(dict(block_size=16, max_num_seqs=4, max_model_len=128), **kw))
+        got = eng.generate(prompts, SamplingParams(max_new_tokens=12))
+        assert got == want, kw
+        assert core.cache.num_free_pages() == eng.config.usable_pages and core.cache.slots.num_free == eng.config.max_num_seqs
+
+
+def test_chunk_count_and_first_token_step():
+    """ceil(T / chunk) portions; the first token comes from the step that ends the prompt
+    (reference: jllm/engine/engine.py:391-403, tests/test_engine.py:129-186)."""
+    eng, core = make(block_size=16, max_num_seqs=1, max_model_len=128, max_num_batched_tokens=16)
+    eng.add_request(list(range(50)), SamplingParams(max_new_tokens=2))
+    events = drain(eng)
+    assert [len(e) for e in events] == [0, 0, 0, 1, 1]
+    assert [s[0][2] for s in core.steps] == [16, 16, 16, 2, 1] and eng.stats.prefill_portions == 4
+
+
+def test_eos_is_emitted_and_counted():
+    """jllm/engine/engine.py:507-512."""
+    prompt = [5, 6, 7]
+    full = expected(prompt, 10)
+    eos = full[3]
+    eng, _ = make(block_size=4, max_model_len=64)
+    got = eng.generate([prompt], SamplingParams(max_new_tokens=10, eos_id=eos))
+    assert got == [full[:full.index(eos) + 1]]
+
+
+def test_fifo_admission_slots_and_arrival_steps():
+    eng, core = make(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=64)
+    ids = [eng.add_request([i, i + 1, i + 2], SamplingParams(max_new_tokens=2), arrival_step=s)
+           for i, s in ((10, 0), (20, 0), (30, 0), (40, 6))]
+    drain(eng)
+    first_seen = {}
+    for i, s in enumerate(core.steps):
+        for rid, *_ in s:
+            first_seen.setdefault(rid, i)
+    assert first_seen[ids[0]] == first_seen[ids[1]] == 0      # two slots
+    assert first_seen[ids[2]] == 2                            # a slot frees after two tokens each
+    assert first_seen[ids[3]] >= 4                            # not before its arrival step (idle steps run nothing)
+    assert eng.scheduler.step_index >= 7
+
+
+def test_prefix_cache_decisions():
+    """Adapted from the reference's tests/test_engine.py:83-126, 189-227 and
+    tests/test_scheduler.py:166-243: with 'the last prompt token is always computed' a repeated
+    32-token prompt hits 1 page of 2 and recomputes the other; a prompt sharing only the first
+    page hits exactly 1."""
+    eng, core = make(block_size=16, max_num_seqs=2, max_model_len=128, max_num_batched_tokens=64)
+    prompt = list(range(32))
+    first = eng.generate([prompt], SamplingParams(max_new_tokens=4))
+    assert eng.stats.cache_hit_blocks == 0
+    second = eng.generate([prompt], SamplingParams(max_new_tokens=4))
+    assert second == first and eng.stats.cache_hit_blocks == 1 and eng.stats.cache_hit_tokens == 16
+    assert core.steps[-4][0][1:3] == (16, 16)                 # only the last 16 tokens were run
+    other = prompt[:16] + [90] * 10
+    eng.generate([other], SamplingParams(max_new_tokens=2))
+    assert eng.stats.cache_hit_blocks == 2
+    # a cached and a cold request admitted together: one step holds the cold prompt whole and the
+    # cached one's remainder; generated tokens enter the cache as pages fill (engine.py:476-490)
+    n0 = len(core.steps)
+    eng.generate([prompt, [50] * 20], SamplingParams(max_new_tokens=1))
+    assert [(c, n) for _, c, n, _ in core.steps[n0]] == [(16, 16), (0, 20)]
+    assert eng.stats.cache_hit_blocks == 3
+    long = eng.generate([prompt], SamplingParams(max_new_tokens=20))[0]
+    again = eng.generate([prompt + long[:17]], SamplingParams(max_new_tokens=1))
+    assert core.steps[-1][0][1] == 48 and again == [expected(prompt + long[:17], 1)]
+
+
+def test_requests_that_can_never_fit_are_refused():
+    eng, _ = make(block_size=4, max_num_seqs=2, max_model_len=64, max_prefill_len=32, num_blocks=1 + 5)
+    with pytest.raises(ValueError, match="empty prompt"):
+        eng.add_request([])
+    with pytest.raises(ValueError, match="max_prefill_len=32"):
+        eng.add_request([1] * 33)
+    with pytest.raises(ValueError, match="max_model_len"):
+        eng.add_request([1] * 30, SamplingParams(max_new_tokens=40))
+    with pytest.raises(ValueError, match="needs 6 pages"):
+        eng.add_request([1] * 20, SamplingParams(max_new_tokens=4))
+    with pytest.raises(ValueError, match="vocabulary"):
+        eng.add_request([VOCAB])
+    eng.add_request([1] * 16, SamplingParams(max_new_tokens=4))       # exactly 5 pages: accepted
+    assert drain(eng)
+
+
+def test_decode_without_a_page_preempts_the_newest_request():
+    # 6 pages of 4: two requests of 9 prompt tokens take 3 pages each (12 slots, 9 used); after 3
+    # decoded tokens each needs a 4th page and none is free
+    eng, core = make(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=64, num_blocks=1 + 6,
+                     enable_prefix_cache=False)
+    p0, p1 = list(range(9)), list(range(20, 29))
+    a = eng.add_request(p0, SamplingParams(max_new_tokens=8))
+    b = eng.add_request(p1, SamplingParams(max_new_tokens=8))
+    drain(eng)
+    assert eng.stats.preemptions >= 1
+    assert eng.requests[b].num_preemptions >= 1 and eng.requests[a].num_preemptions == 0   # the newest yields
+    assert eng.requests[a].output_ids == expected(p0, 8) and eng.requests[b].output_ids == expected(p1, 8)
+    # the preempted request was recomputed from position 0: prompt and the tokens it had generated
+    restarts = [s for s in core.steps for rid, c, n, _ in s if rid == b and c == 0]
+    assert len(restarts) >= 2
+    assert core.cache.num_free_pages() == 6
+
+
+def test_prompt_portion_is_shortened_or_postponed_when_pages_are_short():
+    eng, core = make(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=64, num_blocks=1 + 6,
+                     enable_prefix_cache=False)
+    a = eng.add_request(list(range(14)), SamplingParams(max_new_tokens=2))     # 4 pages
+    b = eng.add_request(list(range(30, 44)), SamplingParams(max_new_tokens=2))  # wants 4, only 2 are free
+    drain(eng)
+    assert core.steps[0] == [(a, 0, 14, [13])]                # b is not admitted: its first portion has no room
+    assert eng.requests[a].output_ids == expected(list(range(14)), 2)
+    assert eng.requests[b].output_ids == expected(list(range(30, 44)), 2)
+    assert eng.stats.preemptions == 0
+
+
+def test_lone_request_larger_than_the_free_pages_starts_with_what_fits():
+    eng, core = make(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=64, num_blocks=1 + 6,
+                     max_chunk=64, enable_prefix_cache=False)
+    eng.add_request(list(range(22)), SamplingParams(max_new_tokens=2))          # 6 pages at full length
+    drain(eng)
+    assert sum(n for s in core.steps for _, _, n, _ in s) == 22 + 1
+
+
+def test_baseline_workload_b_under_a_24_token_budget():
+    """5 requests, prompts 1/9/40/64/100 (two share a 32-token prefix), arrivals at steps
+    0, 0, 2, 3, 5, budget 24, 20 new tokens each."""
+    rng = np.random.default_rng(7)
+    shared = rng.integers(0, VOCAB, size=32).tolist()
+    prompts = [rng.integers(0, VOCAB, size=1).tolist(), rng.integers(0, VOCAB, size=9).tolist(),
+               shared + rng.integers(0, VOCAB, size=8).tolist(), shared + rng.integers(0, VOCAB, size=32).tolist(),
+               rng.integers(0, VOCAB, size=100).tolist()]
+    eng, core = make(block_size=16, max_num_seqs=4, max_model_len=128, max_num_batched_tokens=24)
+    got = eng.generate(prompts, SamplingParams(max_new_tokens=20, temperature=0.8, seed=7), arrival_steps=[0, 0, 2, 3, 5])
+    assert got == [expected(p, 20) for p in prompts]
+    assert all(sum(n for _, _, n, _ in s) <= 24 for s in core.steps)
+    mixed = [s for s in core.steps if any(n > 1 for _, _, n, _ in s) and any(n == 1 and c > 0 for _, c, n, _ in s)]
+    assert mixed, "prompt portions never ran beside decoded tokens"
+    # the second sharer arrives one step after the first: only the first common page is full by then
+    assert eng.stats.cache_hit_blocks == 1
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_random_workloads_with_few_pages_finish_right(seed):
+    rng = np.random.default_rng(seed)
+    n = 12
+    prompts = [rng.integers(0, 5, size=int(rng.integers(1, 40))).tolist() for _ in range(n)]
+    new = [int(rng.integers(1, 16)) for _ in range(n)]
+    eng, core = make(block_size=4, max_num_seqs=int(rng.integers(1, 5)), max_model_len=64,
+                     max_num_batched_tokens=int(rng.integers(2, 30)), num_blocks=1 + int(rng.integers(14, 24)))
+    got = eng.generate(prompts, [SamplingParams(max_new_tokens=k) for k in new],
+                       arrival_steps=sorted(int(x) for x in rng.integers(0, 30, size=n)))
+    assert got == [expected(p, k) for p, k in zip(prompts, new)]
+    core.cache.check_invariants()
+    assert core.cache.num_free_pages() == eng.config.usable_pages
