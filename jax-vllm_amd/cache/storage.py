@@ -51,6 +51,10 @@ def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs:
                 own, other = p.cache, plan[p.cache_of].cache
                 if (own.num_kv_heads, own.head_dim) != (other.num_kv_heads, other.head_dim):
                     raise ValueError(f"run {p.run} cannot read run {p.cache_of}'s cache: head shapes differ")
+                if other.window is not None and (own.window is None or own.window > other.window):
+                    raise ValueError(
+                        f"run {p.run} cannot read run {p.cache_of}'s cache: it needs keys that the owner's "
+                        f"window of {other.window} has already given back")
                 mem.k_pages, mem.v_pages, mem.group, mem.writes = owner.k_pages, owner.v_pages, owner.group, False
         if p.state is not None:
             mem.state = torch.zeros((max_num_seqs, *p.state.shape), dtype=_STATE_DTYPES[p.state.dtype], device=device)

@@ -109,23 +109,34 @@ def attention_core(q, k, v, mask):
     return torch.einsum("hqk,hkd->hqd", probs, v)
 
 
-def attention_block(w: dict, p: str, cfg: dict, x: torch.Tensor, positions: torch.Tensor):
+def attention_block(w: dict, p: str, cfg: dict, x: torch.Tensor, positions: torch.Tensor, window=None,
+                    shared_kv=None, return_kv=False):
     """Projections, per-head q/k RMSNorm over D before RoPE, RoPE, causal attention,
     head-major concat, output projection: jllm/model/common.py:114-137; q/k norm
-    :107-111 with the model's rms_norm_eps (jllm/model/weights.py:128-129)."""
+    :107-111 with the model's rms_norm_eps (jllm/model/weights.py:128-129).
+    Beyond the reference, for tests of the engine's generality: ``window`` keeps only the last
+    ``window`` keys visible, ``shared_kv`` makes the block read another block's (k, v)."""
     t = x.shape[0]
     nq, nkv, d = cfg["num_heads"], cfg["num_kv_heads"], cfg["head_dim"]
     q = linear(w[f"{p}.q_proj.weight"], x).reshape(t, nq, d).transpose(0, 1)
-    k = linear(w[f"{p}.k_proj.weight"], x).reshape(t, nkv, d).transpose(0, 1)
-    v = linear(w[f"{p}.v_proj.weight"], x).reshape(t, nkv, d).transpose(0, 1)
     q = rms_norm(w[f"{p}.q_norm.weight"], cfg["rms_norm_eps"], q)
-    k = rms_norm(w[f"{p}.k_norm.weight"], cfg["rms_norm_eps"], k)
     cos, sin = rope_cos_sin(d, cfg["rope_theta"], positions, x.dtype)
     q = apply_rope(q, cos, sin)
-    k = apply_rope(k, cos, sin)
-    out = attention_core(q, k, v, causal_mask(t, t))
+    if shared_kv is None:
+        k = linear(w[f"{p}.k_proj.weight"], x).reshape(t, nkv, d).transpose(0, 1)
+        v = linear(w[f"{p}.v_proj.weight"], x).reshape(t, nkv, d).transpose(0, 1)
+        k = rms_norm(w[f"{p}.k_norm.weight"], cfg["rms_norm_eps"], k)
+        k = apply_rope(k, cos, sin)
+    else:
+        k, v = shared_kv
+    mask = causal_mask(t, t)
+    if window:
+        idx = torch.arange(t)
+        mask = mask & (idx[None, :] > idx[:, None] - window)
+    out = attention_core(q, k, v, mask)
     out = out.transpose(0, 1).reshape(t, nq * d)
-    return linear(w[f"{p}.o_proj.weight"], out)
+    out = linear(w[f"{p}.o_proj.weight"], out)
+    return (out, (k, v)) if return_kv else out
 
 
 def decoder_layer(w: dict, i: int, cfg: dict, h: torch.Tensor, positions: torch.Tensor):
@@ -175,3 +186,27 @@ def greedy_generate(w: dict, cfg: dict, prompt, max_new_tokens: int, eos_id=None
 def softmax_temperature(logits: torch.Tensor, temperature: float) -> torch.Tensor:
     """Distribution that temperature sampling draws from: softmax(logits / T) in float32."""
     return torch.softmax(logits.to(torch.float32) / temperature, dim=-1)
+
+
+def forward_scheduled(w: dict, cfg: dict, token_ids, schedule, windows=None) -> torch.Tensor:
+    """Whole-sequence forward with the layers run in a given order: ``schedule`` is a list of
+    (layer index, index of the earlier entry whose keys/values it reads, or None); ``windows``
+    maps a layer index to its attention window.  With schedule [(0, None), (1, None), ...] and
+    no windows this is ``forward``."""
+    ids = torch.as_tensor(token_ids, dtype=torch.long)
+    positions = torch.arange(ids.shape[0])
+    eps = cfg["rms_norm_eps"]
+    h = embed(w["model.embed_tokens.weight"], ids)
+    kvs = []
+    for layer, cache_of in schedule:
+        p = f"model.layers.{layer}"
+        a, kv = attention_block(
+            w, f"{p}.self_attn", cfg, rms_norm(w[f"{p}.input_layernorm.weight"], eps, h), positions,
+            window=(windows or {}).get(layer), shared_kv=None if cache_of is None else kvs[cache_of], return_kv=True)
+        kvs.append(kv)
+        h = h + a
+        m = rms_norm(w[f"{p}.post_attention_layernorm.weight"], eps, h)
+        h = h + swiglu(w[f"{p}.mlp.gate_proj.weight"], w[f"{p}.mlp.up_proj.weight"], w[f"{p}.mlp.down_proj.weight"], m)
+    h = rms_norm(w["model.norm.weight"], eps, h)
+    head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+    return linear(head, h)

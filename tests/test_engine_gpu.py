@@ -1,0 +1,479 @@
+"""The engine on the GPU against the plain implementation: generation through the entry
+point, scheduling under pressure, graphs, long decoding, first tokens, parts alone, and the
+generality of layers (a schedule that repeats a layer and shares a cache, windows, a toy mixer
+with state of its own registered from here)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import check_logits, check_tokens_follow, make_core, make_folder, plain_of
+from tests.plain import qwen3_plain as P
+from tests.tiny import ALL_TINY, TINY_A, TINY_B, TINY_C
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    return {t["name"]: make_folder(t, tmp_path_factory.mktemp(f"m{t['name']}")) for t in ALL_TINY}
+
+
+def entry(rid, tokens, want=None):
+    from jax_vllm_amd.engine.entries import StepEntry
+
+    return StepEntry(rid, tokens, range(len(tokens)) if want is None else want)
+
+
+# ------------------------------------------------------------------ generation through the entry point
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_greedy_generation_workload_a(folders, dtype):
+    """BASELINE workload A: 3 requests, prompts of 5, 17 and 33 random ids, greedy, 16 new tokens."""
+    from jax_vllm_amd import LLM, SamplingParams
+
+    cfg, w = plain_of(folders["A"])
+    rng = np.random.default_rng(0)
+    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (5, 17, 33)]
+    llm = LLM(folders["A"], dtype=dtype, block_size=TINY_A["page_size"], max_num_seqs=3, max_model_len=64,
+              max_num_batched_tokens=32)
+    got = llm.generate(prompts, SamplingParams(max_new_tokens=16))
+    assert [len(g) for g in got] == [16, 16, 16]
+    for p, g in zip(prompts, got):
+        check_tokens_follow(dtype, cfg, w, p, g)
+    if dtype == "float32":
+        assert got == [P.greedy_generate(w, cfg, p, 16) for p in prompts]
+    # the reference's functional spelling drives the same engine
+    from jax_vllm_amd import add_request, has_work, make_driver, step
+
+    drv = make_driver(folders["A"], max_num_seqs=1, max_model_len=64, block_size=TINY_A["page_size"], dtype=dtype)
+    add_request(drv, prompts[1], SamplingParams(max_new_tokens=16))
+    out = []
+    while has_work(drv):
+        out += [ev.token for ev in step(drv)]
+    assert out == got[1]
+
+
+def test_temperature_generation_workload_b_is_cut_independent(folders):
+    """BASELINE workload B: prompts 1/9/40/64/100 (two share a 32-token prefix), arrivals at steps
+    0,0,2,3,5, budget 24, temperature 0.8, seed 7, 20 new tokens.  The draws are keyed by
+    (seed, request, index), so another budget, batch width or page pool gives the same tokens."""
+    from jax_vllm_amd import LLM, SamplingParams
+
+    cfg, w = plain_of(folders["B"])
+    rng = np.random.default_rng(1)
+    shared = rng.integers(0, cfg["vocab_size"], size=32).tolist()
+    prompts = [rng.integers(0, cfg["vocab_size"], size=1).tolist(), rng.integers(0, cfg["vocab_size"], size=9).tolist(),
+               shared + rng.integers(0, cfg["vocab_size"], size=8).tolist(),
+               shared + rng.integers(0, cfg["vocab_size"], size=32).tolist(),
+               rng.integers(0, cfg["vocab_size"], size=100).tolist()]
+    sp = SamplingParams(max_new_tokens=20, temperature=0.8, seed=7)
+    base = dict(dtype="fp32", block_size=16, max_model_len=128)
+    a = LLM(folders["B"], max_num_seqs=4, max_num_batched_tokens=24, **base)
+    got = a.generate(prompts, sp, arrival_steps=[0, 0, 2, 3, 5])
+    assert a.stats.cache_hit_blocks >= 1 and a.stats.max_batched_tokens <= 24
+    b = LLM(folders["B"], max_num_seqs=1, max_num_batched_tokens=2048, enable_prefix_cache=False, **base)
+    assert b.generate(prompts, sp) == got
+    c = LLM(folders["B"], max_num_seqs=3, max_num_batched_tokens=7, num_blocks=1 + 9, **base)
+    assert c.generate(prompts, sp) == got
+    # sampled tokens are plausible under the plain distribution and not simply greedy
+    greedy = LLM(folders["B"], max_num_seqs=4, max_num_batched_tokens=2048, **base).generate(prompts, SamplingParams(max_new_tokens=20))
+    assert greedy != got
+    for p, g in zip(prompts, got):
+        seq = list(p)
+        for t in g:
+            prob = P.softmax_temperature(P.forward(w, cfg, seq)[-1], 0.8)[t].item()
+            assert prob > 1e-5
+            seq.append(t)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_few_pages_preemption_and_prefix_reuse_give_the_same_tokens(folders, dtype):
+    from jax_vllm_amd import LLM, SamplingParams
+
+    cfg, w = plain_of(folders["C"])
+    rng = np.random.default_rng(2)
+    # every request fits when admitted and grows into one more page while decoding
+    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (60, 62, 30, 28)]
+    sp = SamplingParams(max_new_tokens=24)
+    roomy = LLM(folders["C"], dtype=dtype, block_size=32, max_num_seqs=4, max_model_len=128, max_num_batched_tokens=512,
+                enable_prefix_cache=False, use_hip_graphs=False)
+    want = roomy.generate(prompts, sp)
+    tight = LLM(folders["C"], dtype=dtype, block_size=32, max_num_seqs=4, max_model_len=128, max_num_batched_tokens=48,
+                num_blocks=1 + 6)
+    got = tight.generate(prompts, sp)
+    assert tight.stats.preemptions > 0
+    if dtype == "float32":
+        assert got == want
+    for p, g in zip(prompts, got):
+        check_tokens_follow(dtype, cfg, w, p, g)
+    tight.core.cache.check_invariants()
+    # with room to keep them, full pages of a prompt seen before are found in the cache
+    keep = LLM(folders["C"], dtype=dtype, block_size=32, max_num_seqs=2, max_model_len=128, max_num_batched_tokens=48,
+               num_blocks=1 + 12)
+    first = keep.generate(prompts[:2], sp)
+    again = keep.generate(prompts[:2], sp)
+    assert keep.stats.cache_hit_blocks == 2 and keep.stats.cache_hit_tokens == 64
+    if dtype == "float32":
+        assert first == again == want[:2]
+    for p, g in zip(prompts[:2], again):
+        check_tokens_follow(dtype, cfg, w, p, g)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_replayed_decode_steps_equal_eager_steps(folders, dtype):
+    """A captured decode step is replayed several times with eager work (prompt portions, other
+    batch widths) in between; every replay must give what the eager launches give."""
+    cfg, w = plain_of(folders["B"])
+    rng = np.random.default_rng(3)
+    reqs = {f"r{i}": rng.integers(0, cfg["vocab_size"], size=n).tolist() for i, n in enumerate((60, 41, 75))}
+    eager = make_core(folders["B"], dtype, 16, graphs=False)
+    graph = make_core(folders["B"], dtype, 16, graphs=True, model=eager.model)
+    for core in (eager, graph):
+        for rid in reqs:
+            core.start_request(rid)
+    outs = {id(eager): [], id(graph): []}
+    for core in (eager, graph):
+        core.run([entry(r, t[:20], []) for r, t in reqs.items()])
+        for i in range(20, 40):
+            live = [r for r, t in reqs.items() if i < len(t)]
+            outs[id(core)].append(core.run([entry(r, reqs[r][i:i + 1], [0]) for r in live]).cpu())
+            if i == 30:   # eager work between replays: a prompt portion of a new request, then its end
+                core.start_request("x")
+                core.run([entry("x", reqs["r0"][:13], [12])])
+                core.finish_request("x")
+    assert graph.graph_replays >= 15 and eager.graph_replays == 0
+    for a, b in zip(outs[id(eager)], outs[id(graph)]):
+        torch.testing.assert_close(a, b, rtol=0, atol=0)
+    expected = {r: P.forward(w, cfg, t).numpy() for r, t in reqs.items()}
+    for i, got in zip(range(20, 40), outs[id(graph)]):
+        live = [r for r, t in reqs.items() if i < len(t)]
+        check_logits(dtype, got.numpy(), np.stack([expected[r][i] for r in live]), what=f"position {i}")
+
+
+# ------------------------------------------------------------------ long decoding, first tokens
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("graphs", [False, True])
+def test_long_decoding(folders, dtype, graphs):
+    cfg, w = plain_of(folders["A"])
+    toks = np.random.default_rng(4).integers(0, cfg["vocab_size"], size=300).tolist()
+    want = P.forward(w, cfg, toks).numpy()
+    core = make_core(folders["A"], dtype, TINY_A["page_size"], pages=40, graphs=graphs)
+    core.start_request("a")
+    got = [core.run([entry("a", toks[:9])]).cpu().numpy()]
+    for i in range(9, 300):
+        got.append(core.run([entry("a", toks[i:i + 1])]).cpu().numpy())
+    check_logits(dtype, np.concatenate(got), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("tiny", ALL_TINY, ids=[t["name"] for t in ALL_TINY])
+def test_first_tokens_of_a_sequence(folders, dtype, tiny):
+    cfg, w = plain_of(folders[tiny["name"]])
+    toks = [7, 3, 11, 2, 5]
+    want = P.forward(w, cfg, toks).numpy()
+    core = make_core(folders[tiny["name"]], dtype, tiny["page_size"])
+    for rid, cuts in (("one", [1, 1, 1, 1, 1]), ("two", [1, 2, 2]), ("whole", [5])):
+        core.start_request(rid)
+        got, at = [], 0
+        for n in cuts:
+            got.append(core.run([entry(rid, toks[at:at + n])]).cpu().numpy())
+            at += n
+        check_logits(dtype, np.concatenate(got), want, what=rid)
+
+
+def test_step_function_refuses_bad_input(folders):
+    from jax_vllm_amd.cache import OutOfPages
+
+    core = make_core(folders["A"], "float32", 8, pages=2)
+    core.start_request("a")
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        core.run([entry("a", [256])])
+    with pytest.raises(ValueError, match="wanted place"):
+        core.run([entry("a", [1, 2], [2])])
+    with pytest.raises(OutOfPages):
+        core.run([entry("a", list(range(17)))])
+    assert core.run([entry("a", list(range(16)), [15])]).shape == (1, 256)   # nothing was consumed by the refusals
+    core.cache.check_invariants()
+
+
+# ------------------------------------------------------------------ each part alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_parts_alone(dtype):
+    from jax_vllm_amd.parts import PartSpec, build_part
+
+    g = torch.Generator().manual_seed(11)
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+    hidden, inter, vocab, t = 72, 200, 333, 9
+    x = torch.randn(t, hidden, generator=g)
+
+    norm = build_part("norm", PartSpec("rmsnorm", {"size": hidden, "eps": 1e-4}))
+    wn = 1 + 0.2 * torch.randn(hidden, generator=g)
+    norm.bind({"weight": wn.cuda()}, dtype)
+    h = x.clone().cuda()
+    delta = torch.randn(t, hidden, generator=g).to(dtype)
+    out = norm.add_norm(h, delta.cuda())
+    torch.testing.assert_close(h.cpu(), x + delta.float())
+    torch.testing.assert_close(out.float().cpu(), P.rms_norm(wn, 1e-4, x + delta.float()), **tol)
+    torch.testing.assert_close(norm.forward(x.to(dtype).cuda()).float().cpu(), P.rms_norm(wn, 1e-4, x.to(dtype).float()), **tol)
+
+    mlp = build_part("feed_forward", PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter}))
+    ws = {k: (0.1 * torch.randn(s, generator=g)).to(dtype) for k, s in
+          (("gate_proj.weight", (inter, hidden)), ("up_proj.weight", (inter, hidden)), ("down_proj.weight", (hidden, inter)))}
+    mlp.bind({k: v.cuda() for k, v in ws.items()}, dtype)
+    for rows in (t, 70):   # few rows (streaming kernel) and many (library product)
+        xi = torch.randn(rows, hidden, generator=g).to(dtype)
+        ref = P.swiglu(ws["gate_proj.weight"].float(), ws["up_proj.weight"].float(), ws["down_proj.weight"].float(), xi.float())
+        torch.testing.assert_close(mlp.forward(xi.cuda()).float().cpu(), ref, **tol)
+
+    emb = build_part("embedding", PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": hidden}))
+    table = torch.randn(vocab, hidden, generator=g).to(dtype)
+    emb.bind({"weight": table.cuda()}, dtype)
+    ids = torch.tensor([0, 332, 17], dtype=torch.int32)
+    torch.testing.assert_close(emb.forward(ids.cuda()).cpu(), P.embed(table.float(), ids.long()))
+
+    head = build_part("head", PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": hidden}))
+    head.bind({"weight": table.cuda()}, dtype)
+    xi = torch.randn(5, hidden, generator=g).to(dtype)
+    logits = head.forward(xi.cuda())
+    assert logits.dtype == torch.float32
+    torch.testing.assert_close(logits.cpu(), P.linear(table.float(), xi.float()), **tol)
+
+    rot = build_part("position", PartSpec("rotary", {"head_dim": 48, "theta": 5e5}))
+    ref_inv = 1.0 / (5e5 ** (torch.arange(0, 48, 2, dtype=torch.float32) / 48))
+    torch.testing.assert_close(rot.inverse_frequencies(), ref_inv, rtol=0, atol=0)
+    with pytest.raises(ValueError, match="rotary_dim"):
+        build_part("position", PartSpec("rotary", {"head_dim": 48, "theta": 1e4, "rotary_dim": 50}))
+    with pytest.raises(ValueError, match="no mixer part named"):
+        build_part("mixer", PartSpec("nonexistent", {}))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_part_alone(folders, dtype):
+    """The mixer with its cache, outside any model: two portions of one request and a second
+    request beside it, against the plain attention block."""
+    from jax_vllm_amd.cache import CacheManager
+    from jax_vllm_amd.cache.storage import allocate_memories
+    from jax_vllm_amd.parts import KVCacheSpec, PartSpec, build_part
+    from jax_vllm_amd.parts.model import RunMemoryPlan
+    from jax_vllm_amd.parts.spec import StepContext
+
+    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    hidden, nq, nkv, d, ps = 80, 6, 3, 32, 8
+    g = torch.Generator().manual_seed(12)
+    att = build_part("mixer", PartSpec("gqa_attention", dict(
+        hidden_size=hidden, num_heads=nq, num_kv_heads=nkv, head_dim=d, qk_norm_eps=1e-5,
+        position=PartSpec("rotary", {"head_dim": d, "theta": 1e4}))))
+    ws = {n: ((0.15 * torch.randn(s.shape, generator=g)) if s.role == "matrix" else 1 + 0.1 * torch.randn(s.shape, generator=g))
+          for n, s in att.tensors().items()}
+    ws = {n: v.to(tdt).float() for n, v in ws.items()}
+    att.bind({n: v.to(tdt if att.tensors()[n].role == "matrix" else torch.float32).cuda() for n, v in ws.items()}, tdt)
+    plan = [RunMemoryPlan(0, 0, att.cache_spec(), None, None)]
+    assert att.cache_spec() == KVCacheSpec(nkv, d, None)
+    mem = allocate_memories(plan, [("full",)], 16, ps, 2, tdt, "cuda")[0]
+    cache = CacheManager([("full",)], ps, 16, 2, enable_prefix_cache=False)
+    cfg = dict(num_heads=nq, num_kv_heads=nkv, head_dim=d, rms_norm_eps=1e-5, rope_theta=1e4)
+    xa, xb = torch.randn(21, hidden, generator=g).to(tdt), torch.randn(5, hidden, generator=g).to(tdt)
+    pw = {f"p.{n}": v for n, v in ws.items()}
+    want_a = P.attention_block(pw, "p", cfg, xa.float(), torch.arange(21))
+    want_b = P.attention_block(pw, "p", cfg, xb.float(), torch.arange(5))
+    cache.start("a"), cache.start("b")
+
+    def step(parts):
+        q_lens = [x.shape[0] for _, x in parts]
+        ctxl = [cache.context_len(r) for r, _ in parts]
+        for (r, x) in parts:
+            cache.reserve(r, x.shape[0])
+        i32 = lambda v: torch.tensor(v, dtype=torch.int32).cuda()
+        width = max(len(cache.block_table(r, 0)) for r, _ in parts)
+        ctx = StepContext(
+            num_tokens=sum(q_lens), num_requests=len(parts),
+            positions=i32([c + i for c, q in zip(ctxl, q_lens) for i in range(q)]),
+            token_req=i32([j for j, q in enumerate(q_lens) for _ in range(q)]),
+            cu_seqlens=i32(np.concatenate([[0], np.cumsum(q_lens)]).tolist()), context_lens=i32(ctxl),
+            slot_ids=i32([cache.slot(r) for r, _ in parts]),
+            block_tables=[i32([cache.block_table(r, 0) + [0] * (width - len(cache.block_table(r, 0))) for r, _ in parts])],
+            slot_mappings=[i32([s for r, x in parts for s in cache.slot_mapping(r, 0, x.shape[0])])],
+            page_size=ps, q_lens_host=q_lens, context_lens_host=ctxl, slot_ids_host=[0] * len(parts),
+            max_q_len=max(q_lens), max_kv_len=max(c + q for c, q in zip(ctxl, q_lens)))
+        out = att.forward(torch.cat([x for _, x in parts]).cuda(), ctx, mem)
+        for r, x in parts:
+            cache.commit(r, [0] * x.shape[0])
+        return out.float().cpu()
+
+    tol = dict(rtol=2e-5, atol=2e-5) if dtype == "float32" else dict(rtol=3e-2, atol=3e-2)
+    o1 = step([("a", xa[:13])])
+    o2 = step([("b", xb), ("a", xa[13:20])])
+    o3 = step([("a", xa[20:21])])
+    torch.testing.assert_close(torch.cat([o1, o2[5:], o3]), want_a, **tol)
+    torch.testing.assert_close(o2[:5], want_b, **tol)
+
+
+# ------------------------------------------------------------------ layers as data
+def custom_model(folder, dtype, schedule, windows):
+    """The tiny model's weights under another ModelSpec: the schedule names layers as it likes
+    and some layers get an attention window."""
+    from jax_vllm_amd.config import resolve
+    from jax_vllm_amd.parts import DecoderModel, LayerRun, ModelSpec, PartSpec
+    from jax_vllm_amd.weights.loader import TORCH_DTYPES, target_dtype
+    from jax_vllm_amd.weights.safetensors_io import SafetensorsFile
+
+    arch, cfg, _ = resolve(folder)
+    spec = arch.build_spec(cfg)
+    layers = []
+    for i, ls in enumerate(spec.layers):
+        if i in windows:
+            params = dict(ls.mixer.params, window=windows[i])
+            ls = type(ls)(**{**{f: getattr(ls, f) for f in ls.__dataclass_fields__}, "mixer": PartSpec(ls.mixer.kind, params)})
+        layers.append(ls)
+    kw = {f: getattr(spec, f) for f in spec.__dataclass_fields__}
+    model = DecoderModel(ModelSpec(**dict(kw, layers=layers, schedule=[LayerRun(l, c) for l, c in schedule])))
+    f = SafetensorsFile(folder / "model.safetensors")
+    compute = TORCH_DTYPES[dtype]
+    model.bind({n: f.tensor(n).cuda().to(target_dtype(ts.role, compute)) for n, ts in model.tensor_specs().items()}, compute)
+    return model
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_schedule_repeats_a_layer_shares_a_cache_and_windows(folders, dtype):
+    cfg, w = plain_of(folders["B"])
+    schedule = [(0, None), (1, None), (0, None), (2, 0), (1, None)]   # layer 0 and 1 twice; run 3 reads run 0's cache
+    windows = {1: 24}
+    model = custom_model(folders["B"], dtype, schedule, windows)
+    plan = model.memory_plan()
+    assert [p.cache_of for p in plan] == [None, None, None, 0, None]
+    with pytest.raises(ValueError, match="already given back"):      # all keys wanted of a cache that keeps a window
+        make_core(None, dtype, 16, pages=4, model=custom_model(folders["B"], dtype, [(0, None), (1, None), (2, 1)], windows))
+    core = make_core(None, dtype, 16, pages=24, model=model)
+    assert core.group_keys == [("full",), ("window", 24)]
+    toks = np.random.default_rng(5).integers(0, cfg["vocab_size"], size=150).tolist()
+    want = P.forward_scheduled(w, cfg, toks, schedule, windows).numpy()
+    assert not np.allclose(want, P.forward(w, cfg, toks).numpy(), atol=1e-2)
+    core.start_request("a")
+    got, at = [], 0
+    for n in [31, 2, 40, 1, 1, 17, 50, 3, 5]:
+        got.append(core.run([entry("a", toks[at:at + n])]).cpu().numpy())
+        at += n
+        core.cache.check_invariants()
+    assert at == 150
+    check_logits(dtype, np.concatenate(got), want)
+    # the window group has given pages back, the full group has not
+    assert core.cache.block_table("a", 1)[:6] == [0] * 6 and all(core.cache.block_table("a", 0))
+    core.finish_request("a")
+    assert core.cache.num_free_pages(0) == core.cache.num_free_pages(1) == 24
+
+
+class RunningMeanMixer:
+    """A toy token mixer with state of its own, defined here and registered from here: its
+    output at a token is a projection of the mean of all inputs of the request up to and
+    including that token.  State per request: the running sum (float).  No pages."""
+
+    def __init__(self, hidden_size: int):
+        self.hidden_size = hidden_size
+
+    def tensors(self):
+        from jax_vllm_amd.parts import TensorSpec
+
+        return {"proj.weight": TensorSpec((self.hidden_size, self.hidden_size))}
+
+    def cache_spec(self):
+        return None
+
+    def state_spec(self):
+        from jax_vllm_amd.parts import StateSpec
+
+        return StateSpec((self.hidden_size,), "float32")
+
+    def bind(self, tensors, dtype):
+        self.w = tensors["proj.weight"]
+
+    def forward(self, x, ctx, mem):
+        out = torch.empty_like(x)
+        at = 0
+        for q, c, slot in zip(ctx.q_lens_host, ctx.context_lens_host, ctx.slot_ids_host):
+            xs = x[at:at + q].float()
+            sums = mem.state[slot][None, :] + torch.cumsum(xs, dim=0)
+            mem.state[slot] = sums[-1]
+            counts = torch.arange(c + 1, c + q + 1, device=x.device, dtype=torch.float32)[:, None]
+            out[at:at + q] = ((sums / counts).to(x.dtype) @ self.w.t()).to(x.dtype)
+            at += q
+        return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype):
+    from jax_vllm_amd.config import register_architecture, resolve
+    from jax_vllm_amd.parts import DecoderModel, LayerRun, LayerSpec, ModelSpec, PartSpec, register_part
+    from jax_vllm_amd.weights.loader import TORCH_DTYPES, target_dtype
+
+    register_part("mixer", "running_mean", RunningMeanMixer)
+    hidden, vocab, inter = 48, 120, 96
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5})
+    att = PartSpec("gqa_attention", dict(hidden_size=hidden, num_heads=3, num_kv_heads=1, head_dim=16, qk_norm_eps=1e-5,
+                                         position=PartSpec("rotary", {"head_dim": 16, "theta": 1e4})))
+    toy = PartSpec("running_mean", {"hidden_size": hidden})
+    ffn = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter})
+
+    def build(_cfg):
+        return ModelSpec(
+            vocab_size=vocab, hidden_size=hidden,
+            embedding=PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": hidden}), embedding_prefix="emb.",
+            final_norm=norm, final_norm_prefix="norm.", head=PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": hidden}),
+            head_prefix="head.", tie_head_to_embedding=True,
+            layers=[LayerSpec(f"l{i}.", mixer, ffn, PartSpec("prenorm", {"norm": norm}), "mix.", "ffn.")
+                    for i, mixer in enumerate([toy, att, toy])],
+            schedule=[LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(0)])
+
+    register_architecture("ToyStateModel", lambda c: c, build)
+    arch, cfg, _ = resolve({"architectures": ["ToyStateModel"]})
+    model = DecoderModel(arch.build_spec(cfg))
+    g = torch.Generator().manual_seed(13)
+    compute = TORCH_DTYPES[dtype]
+    w = {n: ((0.2 * torch.randn(ts.shape, generator=g)) if ts.role == "matrix" else 1 + 0.1 * torch.randn(ts.shape, generator=g))
+         .to(torch.bfloat16).float() for n, ts in model.tensor_specs().items()}
+    model.bind({n: v.cuda().to(target_dtype(model.tensor_specs()[n].role, compute)) for n, v in w.items()}, compute)
+    core = make_core(None, dtype, 8, pages=24, seqs=3, model=model)
+    assert [p.state is not None for p in core.plan] == [True, False, True, True]
+    assert not core.cache.prefix_cache                      # state forbids taking pages over
+    assert [m.state.shape for m in core.memories if m.state is not None] == [(3, hidden)] * 3
+
+    def plain(tokens):
+        t = len(tokens)
+        pos = torch.arange(t)
+        c = dict(num_heads=3, num_kv_heads=1, head_dim=16, rms_norm_eps=1e-5, rope_theta=1e4)
+        h = w["emb.weight"][torch.tensor(tokens)]
+        for i in (0, 1, 2, 0):
+            x = P.rms_norm(w[f"l{i}.input_layernorm.weight"], 1e-5, h)
+            if i == 1:
+                a = P.attention_block(w, "l1.mix", c, x, pos)
+            else:
+                a = (torch.cumsum(x, 0) / torch.arange(1, t + 1)[:, None]) @ w[f"l{i}.mix.proj.weight"].T
+            h = h + a
+            m = P.rms_norm(w[f"l{i}.post_attention_layernorm.weight"], 1e-5, h)
+            h = h + P.swiglu(w[f"l{i}.ffn.gate_proj.weight"], w[f"l{i}.ffn.up_proj.weight"], w[f"l{i}.ffn.down_proj.weight"], m)
+        return (P.rms_norm(w["norm.weight"], 1e-5, h) @ w["emb.weight"].T).numpy()
+
+    rng = np.random.default_rng(6)
+    reqs = {r: rng.integers(0, vocab, size=n).tolist() for r, n in (("a", 40), ("b", 23), ("c", 31))}
+    fed = {r: 0 for r in reqs}
+    got = {r: [] for r in reqs}
+    for r in reqs:
+        core.start_request(r)
+    cuts = [[("a", 7)], [("a", 2), ("b", 9)], [("b", 1), ("c", 31), ("a", 1)], [("a", 30), ("b", 13)]]
+    for step in cuts:
+        es = [entry(r, reqs[r][fed[r]:fed[r] + n]) for r, n in step]
+        out = core.run(es).cpu().numpy()
+        at = 0
+        for r, n in step:
+            got[r].append(out[at:at + n])
+            at += n
+            fed[r] += n
+    for r in reqs:
+        assert fed[r] == len(reqs[r])
+        check_logits(dtype, np.concatenate(got[r]), plain(reqs[r]), what=r)
+    # a slot that is given back and taken again starts from zero state
+    core.finish_request("b")
+    core.start_request("d")
+    out = core.run([entry("d", reqs["c"])]).cpu().numpy()
+    check_logits(dtype, out, plain(reqs["c"]), what="d after b")

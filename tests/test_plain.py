@@ -218,3 +218,17 @@ def test_greedy_generate_stops_on_eos_and_counts_it():
     out2 = P.greedy_generate(w, cfg, [5, 6, 7], 6, eos_id=out[2])
     first = out.index(out[2])
     assert out2 == out[: first + 1]
+
+
+def test_forward_scheduled_reduces_to_forward_and_window_is_a_band():
+    cfg = P_cfg(TINY_B)
+    w = make_weights_dict(TINY_B)
+    ids = list(range(3, 30))
+    base = P.forward(w, cfg, ids)
+    plain_order = [(i, None) for i in range(cfg["num_hidden_layers"])]
+    torch.testing.assert_close(P.forward_scheduled(w, cfg, ids, plain_order), base)
+    # a window at least as long as the sequence changes nothing; a short one changes late rows only
+    torch.testing.assert_close(P.forward_scheduled(w, cfg, ids, plain_order, {0: 27, 1: 100}), base)
+    short = P.forward_scheduled(w, cfg, ids, plain_order, {1: 5})
+    torch.testing.assert_close(short[:5], base[:5])
+    assert not torch.allclose(short[10:], base[10:], rtol=1e-3, atol=1e-4)
