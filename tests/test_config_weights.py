@@ -152,3 +152,23 @@ def test_model_spec_rejects_bad_schedules():
         ModelSpec(**dict(kw, schedule=[LayerRun(0, cache_of=1), LayerRun(1)]))
     with pytest.raises(ValueError, match="no cache of its own"):
         ModelSpec(**dict(kw, schedule=[LayerRun(0), LayerRun(1, cache_of=0), LayerRun(0, cache_of=1)]))
+
+
+def test_command_line_keeps_the_reference_option_names(tmp_path, monkeypatch):
+    """jllm/server.py:245-269: --model-path (env JLLM_MODEL_PATH), --max-num-seqs 4,
+    --max-model-len 2048, --max-prefill-len 512, --dtype {bf16,fp32} default bf16."""
+    from jax_vllm_amd.engine import cli
+
+    monkeypatch.setenv("JLLM_MODEL_PATH", "/some/where")
+    a = cli.build_parser().parse_args([])
+    assert (a.model_path, a.max_num_seqs, a.max_model_len, a.max_prefill_len, a.dtype) == ("/some/where", 4, 2048, 512, "bf16")
+    assert cli.parse_ids("1, 2 3") == [1, 2, 3]
+    (tmp_path / "p.txt").write_text("5 6 7\n\n8,9\n")
+    (tmp_path / "p.json").write_text("[[1, 2], [3]]")
+    assert cli.read_prompts(cli.build_parser().parse_args(["--prompt-ids", "4 4", "--prompt-file", str(tmp_path / "p.txt")])) == [[4, 4], [5, 6, 7], [8, 9]]
+    assert cli.read_prompts(cli.build_parser().parse_args(["--prompt-file", str(tmp_path / "p.json")])) == [[1, 2], [3]]
+    # the random-weights mode writes a loadable folder without a GPU
+    (tmp_path / "c.json").write_text(json.dumps(TINY_A["config"]))
+    assert cli.main(["--random-config", str(tmp_path / "c.json"), "--random-seed", "3", "--write-model", str(tmp_path / "m")]) == 0
+    assert (tmp_path / "m" / "config.json").exists() and (tmp_path / "m" / "model.safetensors").exists()
+    assert cli.main([]) == 2
