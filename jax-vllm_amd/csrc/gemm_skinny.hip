@@ -142,6 +142,108 @@ gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Second organisation, for at most 16 rows of x: a block owns one row tile of W, its WK waves
+// split K; per phase of up to KP columns every wave first issues ALL its W loads (NL pieces of
+// 16 bytes per lane, nothing waits on anything), then the block copies the phase's x columns
+// into LDS (MP = 8 or 16 rows; B-operand lanes of rows >= MP read row % MP, their results are
+// never stored), one barrier, and the products run as the weights arrive.  One or two barriers
+// per phase instead of one per 128 columns.
+template <int NL, typename OutT>
+__global__ void __launch_bounds__(1024)
+gemm_skinny_resident_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
+                            int M, int N, int K, long long ldx, long long ldy, int WK, int MP, int KP) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  bf16_t* xs = (bf16_t*)smem;                // [MP][KP + SK_PAD]
+  const int LROW = KP + SK_PAD;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  const int wk = tid >> 6, lane = tid & 63, li = lane & 15, lc = lane >> 4;
+  const int n = blockIdx.x * 16 + li;
+  const bool n_ok = n < N;
+  const bf16_t* wrow = W + (long long)(n_ok ? n : 0) * K + lc * 8;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int SL = NL * 32;                    // columns of one wave per phase; KP == WK * SL
+  const int n_phase = (K + KP - 1) / KP;
+  // rows M..MP-1 stay zero
+  for (int c = tid; c < MP * LROW / 8; c += nthreads) *(bf16x8*)(xs + c * 8) = zero;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  const int xvecs = M * (KP / 8);
+  const bf16_t* xrow_lds = xs + (li % MP) * LROW + wk * SL + lc * 8;
+  for (int p = 0; p < n_phase; ++p) {
+    const int k0 = p * KP + wk * SL;
+    bf16x8 a[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int k = k0 + i * 32 + lc * 8;
+      a[i] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k0 + i * 32) : zero;
+    }
+    __syncthreads();  // zero fill (first phase) or the previous phase's reads are done
+    for (int c = tid; c < xvecs; c += nthreads) {
+      const int m = c / (KP / 8), kc = c - m * (KP / 8);
+      const int k = p * KP + kc * 8;
+      *(bf16x8*)(xs + m * LROW + kc * 8) = k < K ? *(const bf16x8*)(x + (long long)m * ldx + k) : zero;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const bf16x8 b = *(const bf16x8*)(xrow_lds + i * 32);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b, acc, 0, 0, 0);
+    }
+  }
+  __syncthreads();
+  float* red = (float*)smem;
+  if (WK > 1) {
+    *(f32x4*)(red + (wk * 256 + lane * 4)) = acc;
+    __syncthreads();
+  }
+  if (wk == 0) {
+    f32x4 s = acc;
+    for (int w = 1; w < WK; ++w) {
+      const f32x4 t = *(const f32x4*)(red + (w * 256 + lane * 4));
+      s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
+    }
+    const int nb = blockIdx.x * 16 + lc * 4;
+    if (li < M) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (nb + e < N) y[(long long)li * ldy + nb + e] = from_f32<OutT>(s[e]);
+    }
+  }
+}
+
+template <int NL, typename OutT>
+static int launch_resident(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
+                           long long ldy, int WK, hipStream_t stream) {
+  const int MP = M <= 8 ? 8 : 16;
+  const int KP = WK * NL * 32;
+  size_t shmem = (size_t)MP * (KP + SK_PAD) * 2;
+  if (shmem < (size_t)WK * 256 * 4) shmem = (size_t)WK * 256 * 4;
+  if (shmem > 160 * 1024) return (int)hipErrorInvalidValue;
+  if (shmem > 64 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_resident_kernel<NL, OutT>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+      if (e != hipSuccess) return (int)e;
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL((gemm_skinny_resident_kernel<NL, OutT>), dim3((N + 15) / 16), dim3(WK * 64), shmem, stream,
+                     (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, WK, MP, KP);
+  return JV_LAUNCH_CHECK();
+}
+
+template <typename OutT>
+static int dispatch_resident(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
+                             long long ldy, int WK, hipStream_t s) {
+  switch (nl) {
+    case 4: return launch_resident<4, OutT>(y, x, W, M, N, K, ldx, ldy, WK, s);
+    case 8: return launch_resident<8, OutT>(y, x, W, M, N, K, ldx, ldy, WK, s);
+    case 16: return launch_resident<16, OutT>(y, x, W, M, N, K, ldx, ldy, WK, s);
+  }
+  return (int)hipErrorInvalidValue;
+}
+
 static size_t skinny_shmem(int MT, int NKS, int WR, int WK) {
   const size_t xbytes = (size_t)2 * MT * 16 * (WK * NKS * 32 + SK_PAD) * 2;
   const size_t rbytes = WK > 1 ? (size_t)WR * WK * MT * 256 * 4 : 0;
@@ -210,12 +312,20 @@ static void skinny_config(int M, int N, int K, int* wr, int* wk, int* nks) {
 // out_f32: 0 -> y is bf16, 1 -> y is float.  silu: 0 -> x is [M, K] with row stride ldx;
 // 1 -> x is gate_up [M, 2K] (row stride ldx), the product runs on silu(gate) * up, y is bf16.
 // wr, wk, nks: block shape (row tiles, K slices, MFMA steps per iteration); 0 picks them.
+// wr == -1 selects the resident-x organisation (M <= 16, no silu): wk waves, nks in {4, 8, 16}
+// weight pieces per wave and phase.
 extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
                                    long long ldx, long long ldy, int out_f32, int silu, int wr,
                                    int wk, int nks, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
   if (silu && out_f32) return (int)hipErrorInvalidValue;
+  if (wr == -1) {
+    if (M > 16 || silu || wk < 1 || wk > 16) return (int)hipErrorInvalidValue;
+    hipStream_t s = (hipStream_t)stream;
+    return out_f32 ? dispatch_resident<float>(nks, y, x, W, M, N, K, ldx, ldy, wk, s)
+                   : dispatch_resident<bf16_t>(nks, y, x, W, M, N, K, ldx, ldy, wk, s);
+  }
   int cwr, cwk, cnks;
   skinny_config(M, N, K, &cwr, &cwk, &cnks);
   if (wr <= 0) wr = cwr;

@@ -328,6 +328,11 @@ def sample(logits: torch.Tensor, temperature=None, keys=None, out=None) -> torch
 MFMA_ATTENTION_MAX_HEAD_DIM = 256
 
 
+def attn_prefill_rows(head_dim: int) -> int:
+    """Rows (query, head-in-group pairs) of one block of the prefill kernel."""
+    return 128 if head_dim <= 128 else 64
+
+
 def mfma_attention_supported(dtype, head_dim: int, page_size: int) -> bool:
     """The matrix-core kernels take bfloat16, head sizes that are multiples of 16 up to 256 and
     page sizes that are multiples of 8; everything else goes to the generic kernel."""
@@ -358,7 +363,8 @@ def _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlen
 def attn_prefill_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, n_work,
                       nq, nkv, head_dim, scale, window=0) -> None:
     """Causal attention of prompt portions.  ``work`` is int32 [n_work, 2]: (request index, first row)
-    for every block of 64 rows, a row being a (query, head-in-group) pair of one kv head."""
+    for every block of ``attn_prefill_rows(head_dim)`` rows, a row being a (query, head-in-group) pair of one
+    kv head."""
     page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
                              nq, nkv, head_dim)
     _need(work.numel() >= 2 * n_work, "work list shorter than n_work")

@@ -2,7 +2,7 @@
 
 bfloat16 with a head size and page size the matrix-core kernels are built for: requests with
 one token in the step go to the decode kernel (keys shared out to several blocks when few
-requests would leave the chip idle), all others to the prefill kernel in blocks of 64
+requests would leave the chip idle), all others to the prefill kernel in blocks of 128 (or 64)
 (query, head-in-group) rows, heaviest blocks first.  Everything else (float32, other head
 sizes) runs the generic float-math kernel.  The plan depends on the step's lengths and on
 the heads-per-group ratio only, so it is built once per step and shared by all layers.
@@ -16,7 +16,6 @@ import torch
 
 from ..ops import kernels as K
 
-ROWS_PER_BLOCK = 64          # of the prefill kernel
 TARGET_BLOCKS = 512          # about two blocks per compute unit
 MIN_KEYS_PER_SPLIT = 128     # one 32-key tile for each of a block's 4 waves
 
@@ -40,6 +39,7 @@ def decode_splits(n_decode: int, blocks_per_request: int, max_kv_len: int) -> in
 
 def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, device) -> MfmaPlan:
     g = nq // nkv
+    rows_per_block = K.attn_prefill_rows(head_dim)
     prefill, decode = [], []
     max_kv_decode = 1
     for r, (ql, cl) in enumerate(zip(ctx.q_lens_host, ctx.context_lens_host)):
@@ -47,8 +47,8 @@ def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, device) -> MfmaPlan:
             decode.append(r)
             max_kv_decode = max(max_kv_decode, cl + 1)
         else:
-            for m0 in range(0, ql * g, ROWS_PER_BLOCK):
-                last_row = min(ql * g, m0 + ROWS_PER_BLOCK) - 1
+            for m0 in range(0, ql * g, rows_per_block):
+                last_row = min(ql * g, m0 + rows_per_block) - 1
                 prefill.append((cl + last_row // g + 1, r, m0))
     prefill.sort(key=lambda w: -w[0])
     splits = decode_splits(len(decode), nkv * (-(-g // 16)), max_kv_decode) if decode else 1

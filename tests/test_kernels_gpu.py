@@ -352,7 +352,8 @@ def test_mfma_prefill_attention(case):
     scale = 1.0 / math.sqrt(d)
     qs, ks, vs, dev = _mfma_inputs(nq, nkv, d, page_size, reqs)
     g = nq // nkv
-    work = [x for r, (c, ql) in enumerate(reqs) for m0 in range(0, ql * g, 64) for x in (r, m0)]
+    rpb = K().attn_prefill_rows(d)
+    work = [x for r, (c, ql) in enumerate(reqs) for m0 in range(0, ql * g, rpb) for x in (r, m0)]
     out = torch.full((dev["n"], nq * d), float("nan"), dtype=torch.bfloat16).cuda()
     K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
                           dev["ctx"], torch.tensor(work, dtype=torch.int32).cuda(), len(work) // 2, nq, nkv, d,
@@ -436,7 +437,7 @@ def test_mfma_attention_ignores_garbage_past_the_context():
     ref = _mfma_reference(qs, ks, vs, reqs, scale, None, nq, d)
     out = torch.zeros(dev["n"], nq * d, dtype=torch.bfloat16).cuda()
     K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
-                          dev["ctx"], torch.tensor([0, 0, 0, 64], dtype=torch.int32).cuda(), 2, nq, nkv, d, scale)
+                          dev["ctx"], torch.tensor([0, 0], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
     K().attn_decode_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
                          dev["ctx"], torch.tensor([1], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
     torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
