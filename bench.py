@@ -101,6 +101,8 @@ def main():
                     help="run only the first layers of the 36 (reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="measure the headline batch only")
+    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
+                    help="run one phase alone and print its result (for profiling)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -117,7 +119,7 @@ def main():
     cfg["num_hidden_layers"] = layers
     vocab = cfg["vocab_size"]
     rng = np.random.default_rng(0)
-    max_batch = args.batch if args.skip_points else max(64, args.batch)
+    max_batch = args.batch if (args.skip_points or args.only) else max(64, args.batch)
     block = 16
     llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=max_batch,
               max_model_len=MAX_CONTEXT, num_blocks=1 + max_batch * (-(-(PROMPT_LEN + 2 * 1024) // block)),
@@ -125,6 +127,16 @@ def main():
     itemsize = 2 if args.dtype == "bf16" else 4
     wbytes, per_layer_params = weight_bytes(cfg, layers, itemsize)
     kv_per_token = llm.core.kv_bytes_per_token
+
+    if args.only == "prefill":
+        pre_s = measure_prefill(llm, rng, vocab)
+        print(json.dumps({"prefill_ms": round(pre_s * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}), flush=True)
+        return
+    if args.only == "decode":
+        tps, step_s, mean_ctx = measure_decode(llm, args.batch, args.steps, args.warmup, rng, vocab)
+        print(json.dumps({"decode_tokens_per_s": round(tps, 1), "ms_per_step": round(step_s * 1e3, 4),
+                          "batch": args.batch, "mean_context": round(mean_ctx, 1), "layers": layers}), flush=True)
+        return
 
     # prefill of 2,048 tokens
     pre_s = measure_prefill(llm, rng, vocab)

@@ -43,6 +43,7 @@ class RequestCache:
     tables: list = field(default_factory=list)     # per group: page id per page index (NULL_PAGE once released)
     hashes: list = field(default_factory=list)     # chain hashes of the full pages hashed so far (full group)
     num_cached_tokens: int = 0                     # tokens taken over from the prefix cache at start
+    versions: list = field(default_factory=list)   # per group: bumped whenever the table changes
 
     @property
     def context_len(self) -> int:
@@ -106,7 +107,8 @@ class CacheManager:
         token.  Returns the number of tokens taken over (a multiple of the page size)."""
         if request_id in self.requests:
             raise KeyError(f"request {request_id!r} already started")
-        rc = RequestCache(request_id, self.slots.acquire(), tables=[[] for _ in self.groups])
+        rc = RequestCache(request_id, self.slots.acquire(), tables=[[] for _ in self.groups],
+                          versions=[0] * len(self.groups))
         self.new_slots.append(rc.slot)
         self.requests[request_id] = rc
         if self.prefix_cache and prompt is not None and len(prompt) > 1:
@@ -136,9 +138,11 @@ class CacheManager:
         for g, n in zip(self.groups, need):
             if g.pool.num_free < n:
                 raise OutOfPages(f"group {g.key}: {n} pages needed, {g.pool.num_free} free")
-        for g, table, n in zip(self.groups, rc.tables, need):
+        for gi, (g, table, n) in enumerate(zip(self.groups, rc.tables, need)):
             for _ in range(n):
                 table.append(g.pool.allocate())
+            if n:
+                rc.versions[gi] += 1
 
     def slot_mapping(self, request_id, group: int, num_new_tokens: int) -> list:
         """Flat cache slot (page * page_size + offset) of each of the next tokens."""
@@ -154,6 +158,10 @@ class CacheManager:
 
     def block_table(self, request_id, group: int) -> list:
         return self.requests[request_id].tables[group]
+
+    def table_version(self, request_id, group: int) -> int:
+        """Changes whenever the request's block table of this group does."""
+        return self.requests[request_id].versions[group]
 
     def slot(self, request_id) -> int:
         return self.requests[request_id].slot
@@ -171,7 +179,7 @@ class CacheManager:
                 h = chain_hash(rc.hashes[-1] if rc.hashes else b"", rc.tokens[i * ps:(i + 1) * ps])
                 pool.register_hash(table[i], h)
                 rc.hashes.append(h)
-        for g, table in zip(self.groups, rc.tables):
+        for gi, (g, table) in enumerate(zip(self.groups, rc.tables)):
             w = g.window
             if w is None:
                 continue
@@ -182,6 +190,8 @@ class CacheManager:
             g.pool.release([table[i] for i in gone])
             for i in gone:
                 table[i] = NULL_PAGE
+            if gone:
+                rc.versions[gi] += 1
 
     def finish(self, request_id) -> None:
         """Give back everything the request holds."""

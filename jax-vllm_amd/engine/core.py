@@ -51,10 +51,18 @@ class _DecodeGraph:
             at += size
         self.host_tensor = torch.zeros(at, dtype=torch.int32, pin_memory=True)
         self.host = self.host_tensor.numpy()
+        a, b = self.offsets["token_req"]
+        self.host[a:b] = np.arange(rb, dtype=np.int32)
+        a, b = self.offsets["cu"]
+        self.host[a:b] = np.arange(rb + 1, dtype=np.int32)
+        a, b = self.offsets["rows"]
+        self.host[a:b] = np.arange(rb, dtype=np.int32)
+        self.row_signature = [[None] * rb for _ in range(n_groups)]   # (request, table version) per table row
         self.dev = torch.zeros(at, dtype=torch.int32, device=device)
         self.graph = None
         self.logits = None
         self.ctx = None
+        self.copied = None   # event recorded after each upload of the pinned buffer
 
     def segment(self, host, name):
         a, b = self.offsets[name]
@@ -154,31 +162,46 @@ class EngineCore:
         r = len(entries)
         rb = _bucket(r)
         n_groups = len(self.group_keys)
-        tables = [[cache.block_table(e.request_id, g) for e in entries] for g in range(n_groups)]
-        widths = tuple(_bucket(max(len(t) for t in tables[g]), 8) for g in range(n_groups))
+        widths = tuple(_bucket(max(len(cache.block_table(e.request_id, g)) for e in entries), 8)
+                       for g in range(n_groups))
         key = (rb, widths)
         g = self._graphs.get(key)
         if g is None:
             g = self._graphs[key] = _DecodeGraph(rb, widths, n_groups, self.device)
+        if g.copied is not None:
+            g.copied.synchronize()   # the previous step's upload has left the pinned buffer
         host = g.host
-        host[:] = 0
         seg = g.segment
-        ctx_lens = [cache.context_len(e.request_id) for e in entries]
+        reqs = [cache.requests[e.request_id] for e in entries]
+        ctx_lens = [rc.context_len for rc in reqs]
+        for name in ("tokens", "positions", "ctx", "slots"):
+            seg(host, name)[r:] = 0
         seg(host, "tokens")[:r] = [int(e.tokens[0]) for e in entries]
         seg(host, "positions")[:r] = ctx_lens
-        seg(host, "token_req")[:] = np.arange(rb, dtype=np.int32)
-        seg(host, "cu")[:] = np.arange(rb + 1, dtype=np.int32)
         seg(host, "ctx")[:r] = ctx_lens
-        seg(host, "slots")[:r] = [cache.slot(e.request_id) for e in entries]
-        seg(host, "rows")[:] = np.arange(rb, dtype=np.int32)
+        seg(host, "slots")[:r] = [rc.slot for rc in reqs]
         for gi in range(n_groups):
             sm = seg(host, f"slot_mapping{gi}")
-            sm[:] = -1
-            sm[:r] = [cache.slot_mapping(e.request_id, gi, 1)[0] for e in entries]
+            sm[r:] = -1
+            sm[:r] = [rc.tables[gi][c // ps] * ps + c % ps for rc, c in zip(reqs, ctx_lens)]
+            # block-table rows are rewritten only when the request in the row or its table changed
             bt = seg(host, f"table{gi}").reshape(rb, widths[gi])
-            for i, t in enumerate(tables[gi]):
-                bt[i, :len(t)] = t
+            sig = g.row_signature[gi]
+            for i, rc in enumerate(reqs):
+                s = (rc.request_id, rc.versions[gi])
+                if sig[i] != s:
+                    t = rc.tables[gi]
+                    bt[i, :len(t)] = t
+                    bt[i, len(t):] = 0
+                    sig[i] = s
+            for i in range(r, rb):
+                if sig[i] is not None:
+                    bt[i, :] = 0
+                    sig[i] = None
         g.dev.copy_(g.host_tensor, non_blocking=True)
+        if g.copied is None:
+            g.copied = torch.cuda.Event()
+        g.copied.record()
         if g.graph is None:
             # first use: run the launches eagerly (this is the step's result), then record them
             ctx = g.context(ps, self.page_size * max(widths, default=1))

@@ -142,6 +142,11 @@ class LLM(Engine):
         self.sampler = Sampler(self.core.device)
         super().__init__(config, self.core.cache, self.core.run, self.sampler.sample, self.core.vocab_size)
 
+    def step(self) -> list:
+        events = super().step()
+        self.stats.graph_replays = self.core.graph_replays
+        return events
+
 
 # ---- the reference's functional spelling ------------------------------------------------
 def make_driver(model, max_num_seqs: int, max_model_len: int, max_prefill_len: Optional[int] = None,

@@ -17,7 +17,7 @@ class SamplingParams:
     seed: Optional[int] = None        # None: the engine's seed combined with the request id
 
 
-@dataclass
+@dataclass(eq=False)   # requests are compared by identity: queue membership tests stay O(1) per item
 class Request:
     request_id: int
     prompt_ids: list

@@ -94,19 +94,28 @@ class Scheduler:
             for g in range(len(reserved)):
                 reserved[g] += need[g]
 
+        def fits(need):
+            return all(g.pool.num_free - r >= n for g, n, r in zip(cache.groups, need, reserved))
+
         # 1. decodes (one token each), oldest first; a decode without a page preempts the newest
+        preempted_any = False
         for req in list(self.running):
-            if req not in self.running or req.num_remaining != 1 or budget <= 0:
+            if budget <= 0:
+                break
+            if req.num_remaining != 1 or (preempted_any and req not in self.running):
                 continue
-            while not cache.can_store(req.request_id, 1, reserve=reserved):
+            need = cache.pages_needed(req.request_id, 1)
+            while not fits(need):
                 victim = self._newest_unscheduled(out)
                 if victim is None:
                     break
                 self._preempt(victim, out)
+                preempted_any = True
                 if victim is req:
                     break
-            if req in self.running and cache.can_store(req.request_id, 1, reserve=reserved):
-                take(req, 1)
+            if (not preempted_any or req in self.running) and fits(need):
+                for g in range(len(reserved)):
+                    reserved[g] += need[g]
                 out.items.append(ScheduledItem(req, 1, True))
                 budget -= 1
 

@@ -132,9 +132,10 @@ def _attn_source() -> Path:
 def build_all(force: bool = True) -> None:
     """Compile the core library and the attention library of every supported head size."""
     _ensure("libjvamd", _core_sources(), [], force)
-    if _attn_source().exists():
-        for d in ATTN_HEAD_DIMS:
-            _ensure(f"libjvamd_attn_d{d}", [_attn_source()], [f"-DJV_HEAD_DIM={d}"], force)
+    workers = max(1, min(int(os.environ.get("MAX_JOBS", "0")) or os.cpu_count() or 4, 16))
+    with ThreadPoolExecutor(workers) as ex:
+        list(ex.map(lambda d: _ensure(f"libjvamd_attn_d{d}", [_attn_source()], [f"-DJV_HEAD_DIM={d}"], force),
+                    ATTN_HEAD_DIMS))
 
 
 def _load(name: str, sources: list[Path], defines: list[str]) -> ctypes.CDLL:
@@ -154,7 +155,8 @@ def _load(name: str, sources: list[Path], defines: list[str]) -> ctypes.CDLL:
 
 def core() -> ctypes.CDLL:
     """The core kernel library (built at first use if missing or stale)."""
-    return _load("libjvamd", _core_sources(), [])
+    lib = _handles.get("libjvamd")
+    return lib if lib is not None else _load("libjvamd", _core_sources(), [])
 
 
 def attention(head_dim: int) -> ctypes.CDLL:
@@ -163,4 +165,6 @@ def attention(head_dim: int) -> ctypes.CDLL:
         raise KernelLibraryError(
             f"no MFMA attention kernel for head size {head_dim}: supported are multiples of 16 up to {ATTN_HEAD_DIMS[-1]}"
         )
-    return _load(f"libjvamd_attn_d{head_dim}", [_attn_source()], [f"-DJV_HEAD_DIM={head_dim}"])
+    name = f"libjvamd_attn_d{head_dim}"
+    lib = _handles.get(name)
+    return lib if lib is not None else _load(name, [_attn_source()], [f"-DJV_HEAD_DIM={head_dim}"])
