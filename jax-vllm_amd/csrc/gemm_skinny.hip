@@ -326,6 +326,12 @@ extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M,
     return out_f32 ? dispatch_resident<float>(nks, y, x, W, M, N, K, ldx, ldy, wk, s)
                    : dispatch_resident<bf16_t>(nks, y, x, W, M, N, K, ldx, ldy, wk, s);
   }
+  if (wr == 0 && wk == 0 && nks == 0 && M <= 2 && !silu && K >= 2048 && K <= 4096 && N >= 8192) {
+    // one or two rows against a wide matrix: the resident-x organisation measured ~10 % faster
+    hipStream_t s = (hipStream_t)stream;
+    return out_f32 ? dispatch_resident<float>(16, y, x, W, M, N, K, ldx, ldy, 8, s)
+                   : dispatch_resident<bf16_t>(16, y, x, W, M, N, K, ldx, ldy, 8, s);
+  }
   int cwr, cwk, cnks;
   skinny_config(M, N, K, &cwr, &cwk, &cnks);
   if (wr <= 0) wr = cwr;
