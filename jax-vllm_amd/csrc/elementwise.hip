@@ -135,7 +135,29 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* __restrict__ x,
 }
 
 // ---------------------------------------------------------------- SiLU-mul
-// out[t, j] = silu(gu[t, j]) * gu[t, inter + j], silu(x) = x / (1 + exp(-x)), in float.
+// out[t, j] = silu(gate) * up, silu(x) = x / (1 + exp(-x)), in float.  Two layouts of gu[t, 2*inter]:
+// halves (gate = gu[t, j], up = gu[t, inter + j]) or interleaved (gate = gu[t, 2j], up = gu[t, 2j+1]).
+// Interleaved layout (gate and up alternate along the row): out[t, j] = silu(gu[t, 2j]) * gu[t, 2j+1];
+// each thread takes two outputs (4 inputs) when inter is even.
+template <typename T>
+__global__ void silu_mul_pairs_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
+  const long long t = blockIdx.y;
+  const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 2;
+  if (j >= inter) return;
+  const T* gp = gu + t * 2 * inter + 2 * j;
+  T* op = out + t * inter + j;
+  if (j + 1 < inter && (inter & 1) == 0) {
+    const float4 v = load4<T>(gp);
+    op[0] = from_f32<T>(v.x / (1.f + expf(-v.x)) * v.y);
+    op[1] = from_f32<T>(v.z / (1.f + expf(-v.z)) * v.w);
+  } else {
+    for (int e = 0; e < 2 && j + e < inter; ++e) {
+      const float g = to_f32(gp[2 * e]), u = to_f32(gp[2 * e + 1]);
+      op[e] = from_f32<T>(g / (1.f + expf(-g)) * u);
+    }
+  }
+}
+
 // grid (column blocks, tokens); each thread takes 4 neighbouring columns when inter % 4 == 0.
 template <typename T, int VEC>
 __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
@@ -197,13 +219,16 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \
   extern "C" int jv_silu_mul_##SUF(void* out, const void* gu, long long n_tokens, int inter,        \
-                                   void* stream) {                                                  \
+                                   int interleaved, void* stream) {                                 \
     if (n_tokens <= 0 || inter <= 0) return 0;                                                      \
     for (long long t0 = 0; t0 < n_tokens; t0 += 65535) { /* grid.y limit */                         \
       const unsigned ny = (unsigned)(n_tokens - t0 < 65535 ? n_tokens - t0 : 65535);                \
       T* o = (T*)out + t0 * inter;                                                                  \
       const T* g = (const T*)gu + t0 * 2 * inter;                                                   \
-      if (inter % 4 == 0) {                                                                         \
+      if (interleaved) {                                                                            \
+        hipLaunchKernelGGL((silu_mul_pairs_kernel<T>), dim3(((inter + 1) / 2 + 255) / 256, ny),     \
+                           dim3(256), 0, (hipStream_t)stream, o, g, inter);                         \
+      } else if (inter % 4 == 0) {                                                                         \
         hipLaunchKernelGGL((silu_mul_kernel<T, 4>), dim3((inter / 4 + 255) / 256, ny), dim3(256),   \
                            0, (hipStream_t)stream, o, g, inter);                                    \
       } else {                                                                                      \

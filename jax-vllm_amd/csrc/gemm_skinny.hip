@@ -13,9 +13,9 @@
 // operands from there.  Partial tiles of the WK slices are added through LDS in a fixed
 // order, so a result does not depend on M, on the grid or on timing.
 //
-// Optional prologue for the feed-forward's second product: x = silu(gate) * up computed
-// (in float) from gate_up[M, 2K] while the chunk is copied into LDS, which saves the
-// activation kernel and its round trip.
+// Optional epilogue for the feed-forward's first product: when the rows of W alternate gate and
+// up rows, y[m, j] = silu(x.W[2j]) * (x.W[2j+1]) straight from the float accumulators (a lane
+// holds both numbers of a pair), which saves the activation kernel and its round trip.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -23,7 +23,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define SK_PAD 8  // bf16 elements of padding per LDS row (keeps 16-byte reads of 16 rows off the same banks)
 
-template <int MT, int NKS, typename OutT, bool SILU>
+template <int MT, int NKS, typename OutT, bool PAIRS>
 __global__ void __launch_bounds__(1024)
 gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
                    int M, int N, int K, long long ldx, long long ldy, int WR, int WK) {
@@ -52,16 +52,7 @@ gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     const int m = c / (KCB / 8), kc = c - m * (KCB / 8);
     const int k = it * KCB + kc * 8;
     if (k >= K) return zero;
-    if (!SILU) return *(const bf16x8*)(x + (long long)m * ldx + k);
-    const bf16_t* g = x + (long long)m * ldx + k;
-    const bf16x8 gv = *(const bf16x8*)g, uv = *(const bf16x8*)(g + K);
-    bf16x8 r;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float gf = (float)gv[e], uf = (float)uv[e];
-      r[e] = (bf16_t)(gf / (1.f + expf(-gf)) * uf);
-    }
-    return r;
+    return *(const bf16x8*)(x + (long long)m * ldx + k);
   };
   auto store_x_piece = [&](int buf, int c, bf16x8 v) {
     const int m = c / (KCB / 8), kc = c - m * (KCB / 8);
@@ -135,9 +126,17 @@ gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     const int m = mt * 16 + li;
     const int nb = (blockIdx.x * WR + wr) * 16 + lc * 4;
     if (m < M) {
+      if (PAIRS) {
+        // rows of W alternate gate, up: column pair (2j, 2j+1) -> y[m, j] = silu(gate) * up
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (nb + e < N) y[(long long)m * ldy + nb + e] = from_f32<OutT>(s[e]);
+        for (int e = 0; e < 4; e += 2)
+          if (nb + e + 1 < N)
+            y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(s[e] / (1.f + expf(-s[e])) * s[e + 1]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (nb + e < N) y[(long long)m * ldy + nb + e] = from_f32<OutT>(s[e]);
+      }
     }
   }
 }
@@ -250,44 +249,44 @@ static size_t skinny_shmem(int MT, int NKS, int WR, int WK) {
   return xbytes > rbytes ? xbytes : rbytes;
 }
 
-template <int MT, int NKS, typename OutT, bool SILU>
+template <int MT, int NKS, typename OutT, bool PAIRS>
 static int launch_skinny(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
                          long long ldy, int WR, int WK, hipStream_t stream) {
   const size_t shmem = skinny_shmem(MT, NKS, WR, WK);
   if (shmem > 64 * 1024) {
     static bool raised = false;  // per instantiation
     if (!raised) {
-      hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NKS, OutT, SILU>,
+      hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<MT, NKS, OutT, PAIRS>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
       if (e != hipSuccess) return (int)e;
       raised = true;
     }
   }
   const int blocks = (N + 16 * WR - 1) / (16 * WR);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NKS, OutT, SILU>), dim3(blocks), dim3(WR * WK * 64), shmem,
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, NKS, OutT, PAIRS>), dim3(blocks), dim3(WR * WK * 64), shmem,
                      stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, WR, WK);
   return JV_LAUNCH_CHECK();
 }
 
-template <int NKS, typename OutT, bool SILU>
+template <int NKS, typename OutT, bool PAIRS>
 static int dispatch_mt(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
                        long long ldy, int WR, int WK, hipStream_t s) {
   switch ((M + 15) / 16) {
-    case 1: return launch_skinny<1, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 2: return launch_skinny<2, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 3: return launch_skinny<3, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 4: return launch_skinny<4, NKS, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 1: return launch_skinny<1, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 2: return launch_skinny<2, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 3: return launch_skinny<3, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 4: return launch_skinny<4, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
   }
   return (int)hipErrorInvalidValue;
 }
 
-template <typename OutT, bool SILU>
+template <typename OutT, bool PAIRS>
 static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, int N, int K,
                         long long ldx, long long ldy, int WR, int WK, hipStream_t s) {
   switch (nks) {
-    case 2: return dispatch_mt<2, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 4: return dispatch_mt<4, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 8: return dispatch_mt<8, OutT, SILU>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 2: return dispatch_mt<2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 4: return dispatch_mt<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 8: return dispatch_mt<8, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
   }
   return (int)hipErrorInvalidValue;
 }
@@ -309,24 +308,26 @@ static void skinny_config(int M, int N, int K, int* wr, int* wk, int* nks) {
   *wr = WR; *wk = WK; *nks = NKS;
 }
 
-// out_f32: 0 -> y is bf16, 1 -> y is float.  silu: 0 -> x is [M, K] with row stride ldx;
-// 1 -> x is gate_up [M, 2K] (row stride ldx), the product runs on silu(gate) * up, y is bf16.
+// out_f32: 0 -> y is bf16, 1 -> y is float.  x is [M, K] with row stride ldx.
+// silu_pairs: 1 -> the rows of W alternate gate and up rows and y[m, j] =
+//      silu(x.W[2j]) * (x.W[2j+1]) is bf16 [M, N/2] (the feed-forward's first product with its
+//      activation as epilogue).
 // wr, wk, nks: block shape (row tiles, K slices, MFMA steps per iteration); 0 picks them.
 // wr == -1 selects the resident-x organisation (M <= 16, no silu): wk waves, nks in {4, 8, 16}
 // weight pieces per wave and phase.
 extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
-                                   long long ldx, long long ldy, int out_f32, int silu, int wr,
+                                   long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
                                    int wk, int nks, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
-  if (silu && out_f32) return (int)hipErrorInvalidValue;
+  if (silu_pairs && (out_f32 || N % 2 != 0 || wr == -1)) return (int)hipErrorInvalidValue;
   if (wr == -1) {
-    if (M > 16 || silu || wk < 1 || wk > 16) return (int)hipErrorInvalidValue;
+    if (M > 16 || wk < 1 || wk > 16) return (int)hipErrorInvalidValue;
     hipStream_t s = (hipStream_t)stream;
     return out_f32 ? dispatch_resident<float>(nks, y, x, W, M, N, K, ldx, ldy, wk, s)
                    : dispatch_resident<bf16_t>(nks, y, x, W, M, N, K, ldx, ldy, wk, s);
   }
-  if (wr == 0 && wk == 0 && nks == 0 && M <= 2 && !silu && K >= 2048 && K <= 4096 && N >= 8192) {
+  if (wr == 0 && wk == 0 && nks == 0 && M <= 2 && !silu_pairs && K >= 2048 && K <= 4096 && N >= 8192) {
     // one or two rows against a wide matrix: the resident-x organisation measured ~10 % faster
     hipStream_t s = (hipStream_t)stream;
     return out_f32 ? dispatch_resident<float>(16, y, x, W, M, N, K, ldx, ldy, 8, s)
@@ -341,7 +342,7 @@ extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M,
   if (wr * wk > 16 || (nks != 2 && nks != 4 && nks != 8)) return (int)hipErrorInvalidValue;
   if (skinny_shmem(MT, nks, wr, wk) > 160 * 1024) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
-  if (silu) return dispatch_nks<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
+  if (silu_pairs) return dispatch_nks<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
   if (out_f32) return dispatch_nks<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
   return dispatch_nks<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
 }

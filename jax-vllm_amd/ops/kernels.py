@@ -132,8 +132,9 @@ def cast_rows(x: torch.Tensor, dtype: torch.dtype, rows=None) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- activation
-def silu_mul(gate_up: torch.Tensor, out=None) -> torch.Tensor:
-    """out[t, j] = silu(gate_up[t, j]) * gate_up[t, I + j] for gate_up of width 2 I."""
+def silu_mul(gate_up: torch.Tensor, out=None, interleaved: bool = False) -> torch.Tensor:
+    """out[t, j] = silu(gate) * up for gate_up of width 2 I: gate = gate_up[t, j], up =
+    gate_up[t, I + j], or with ``interleaved`` gate = gate_up[t, 2j], up = gate_up[t, 2j + 1]."""
     _dev(gate_up)
     n, two_i = gate_up.shape
     _need(two_i % 2 == 0, "gate_up must have an even width")
@@ -143,7 +144,8 @@ def silu_mul(gate_up: torch.Tensor, out=None) -> torch.Tensor:
     _dev(out)
     _need(out.shape == (n, inter) and out.dtype == gate_up.dtype, "out must be [tokens, I] of gate_up's type")
     fn = getattr(library.core(), f"jv_silu_mul_{_suffix(gate_up.dtype)}")
-    _check(fn(_ptr(out), _ptr(gate_up), c_longlong(n), c_int(inter), _stream()), "silu_mul")
+    _check(fn(_ptr(out), _ptr(gate_up), c_longlong(n), c_int(inter), c_int(1 if interleaved else 0), _stream()),
+           "silu_mul")
     return out
 
 
@@ -250,28 +252,31 @@ SKINNY_MAX_ROWS = 64
 SKINNY_AUTO_ROWS = 16   # up to here ``linear`` prefers the streaming kernel to the library
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_gate_up: bool = False,
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_pairs: bool = False,
                 block_shape=(0, 0, 0), out=None) -> torch.Tensor:
     """x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w [N, K]: the weight-streaming
-    product of decode steps.  With ``silu_gate_up`` x is gate_up [M, 2K] and the product runs on
-    silu(gate) * up (bfloat16 output only).  Output bfloat16 or float32.  ``block_shape``:
-    (row tiles, K slices, MFMA steps per iteration) of a block, zeros: chosen from the shape."""
+    product of decode steps.  With ``silu_pairs`` the rows of w alternate gate and up rows and
+    the result is silu(x.w[2j]) * (x.w[2j+1]), bfloat16 [M, N/2].  Output bfloat16 or float32.
+    ``block_shape``: (row tiles, K slices, MFMA steps per iteration) of a block, zeros: chosen
+    from the shape; (-1, waves, pieces) selects the organisation with x resident in LDS."""
     _dev(x, w, out)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     m = x.shape[0]
     n, k = w.shape
-    _need(x.dim() == 2 and x.shape[1] == (2 * k if silu_gate_up else k), "inner sizes differ")
+    _need(x.dim() == 2 and x.shape[1] == k, "inner sizes differ")
     _need(m <= SKINNY_MAX_ROWS, f"gemm_skinny takes at most {SKINNY_MAX_ROWS} rows")
     _need(k % 8 == 0, "the inner size must be a multiple of 8")
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
-    _need(not (silu_gate_up and out_dtype != torch.bfloat16), "the silu prologue writes bfloat16 only")
+    _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
+          "the silu epilogue writes bfloat16, needs an even number of rows of w and the chunked organisation")
+    n_out = n // 2 if silu_pairs else n
     if out is None:
-        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
-    _need(out.shape == (m, n) and out.dtype == out_dtype, "out must be [M, N] of the output type")
+        out = torch.empty((m, n_out), dtype=out_dtype, device=x.device)
+    _need(out.shape == (m, n_out) and out.dtype == out_dtype, "out must be [M, N] (or [M, N/2]) of the output type")
     _check(
         library.core().jv_gemm_skinny_bf16(
-            _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.shape[1]), c_longlong(n),
-            c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_gate_up else 0),
+            _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.shape[1]), c_longlong(n_out),
+            c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_pairs else 0),
             c_int(block_shape[0]), c_int(block_shape[1]), c_int(block_shape[2]), _stream()),
         "gemm_skinny",
     )

@@ -1,6 +1,8 @@
 """Gated feed-forward (SwiGLU).  Reference: ``jllm/model/common.py:69-76``:
-``down( silu(gate(x)) * up(x) )``, no biases.  gate and up are one matrix product
-against the row-concatenated weight; the activation runs in float."""
+``down( silu(gate(x)) * up(x) )``, no biases.  gate and up are one matrix product against
+one weight whose rows alternate gate row j, up row j, so that a gate value and its up value
+come out next to each other: for few rows the activation is that product's epilogue, for
+many rows a kernel over adjacent pairs.  The activation runs in float."""
 from __future__ import annotations
 
 import torch
@@ -25,16 +27,16 @@ class GatedMLP:
         }
 
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
-        self.w_gate_up = torch.cat([tensors["gate_proj.weight"], tensors["up_proj.weight"]], dim=0).contiguous()
+        g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        self.w_gate_up = torch.stack([g, u], dim=1).reshape(2 * g.shape[0], g.shape[1]).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
-        gate_up = K.linear(x, self.w_gate_up)
-        if gate_up.shape[0] <= 2 and K.skinny_applies(gate_up, self.w_down):
-            # one or two rows: the activation runs inside the second product's prologue (every
-            # block of that product redoes it, which costs more than a kernel beyond two rows)
-            return K.gemm_skinny(gate_up, self.w_down, gate_up.dtype, silu_gate_up=True)
-        return K.linear(K.silu_mul(gate_up), self.w_down)
+        if K.skinny_applies(x, self.w_gate_up):
+            z = K.gemm_skinny(x, self.w_gate_up, x.dtype, silu_pairs=True)
+        else:
+            z = K.silu_mul(K.linear(x, self.w_gate_up), interleaved=True)
+        return K.linear(z, self.w_down)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

@@ -76,12 +76,16 @@ def test_rmsnorm_last_axis(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("inter", [176, 12288])
+@pytest.mark.parametrize("inter", [176, 12288, 77])
 def test_silu_mul(dtype, inter):
     gu = randn(9, 2 * inter, dtype=dtype, seed=6, scale=3.0)
     out = K().silu_mul(gu)
     g, u = gu.float()[:, :inter], gu.float()[:, inter:]
     torch.testing.assert_close(out.float(), torch.nn.functional.silu(g) * u, **tol(dtype))
+    # gate and up alternating along the row
+    out2 = K().silu_mul(gu, interleaved=True)
+    g2, u2 = gu.float()[:, 0::2], gu.float()[:, 1::2]
+    torch.testing.assert_close(out2.float(), torch.nn.functional.silu(g2) * u2, **tol(dtype))
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 50, 70), (5, 333, 80), (70, 130, 257), (130, 64, 16)])
@@ -484,11 +488,14 @@ def test_gemm_skinny(m, n, k, shape, out_dtype):
         torch.testing.assert_close(one, out[2:3] if m > 2 else out[:1], **exact)
 
 
-@pytest.mark.parametrize("m,inter,n", [(1, 176, 80), (8, 12288, 96), (40, 224, 100)])
-def test_gemm_skinny_silu_prologue(m, inter, n):
-    gu = randn(m, 2 * inter, dtype=torch.bfloat16, seed=32, scale=2.0)
-    w = randn(n, inter, dtype=torch.bfloat16, seed=33, scale=0.3)
-    out = K().gemm_skinny(gu, w, torch.bfloat16, silu_gate_up=True)
-    z = (torch.nn.functional.silu(gu.float()[:, :inter]) * gu.float()[:, inter:]).to(torch.bfloat16)
-    ref = z.double() @ w.double().T
-    torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=2e-2 * math.sqrt(inter) / 4)
+@pytest.mark.parametrize("m,inter,k", [(1, 176, 80), (8, 12288, 96), (40, 224, 104), (16, 1000, 4096)])
+def test_gemm_skinny_silu_epilogue(m, inter, k):
+    """Rows of w alternate gate and up rows; the product comes out as silu(gate) * up."""
+    x = randn(m, k, dtype=torch.bfloat16, seed=32, scale=0.7)
+    wg = randn(inter, k, dtype=torch.bfloat16, seed=33, scale=0.3)
+    wu = randn(inter, k, dtype=torch.bfloat16, seed=34, scale=0.3)
+    w = torch.stack([wg, wu], dim=1).reshape(2 * inter, k).contiguous()
+    out = K().gemm_skinny(x, w, torch.bfloat16, silu_pairs=True)
+    assert out.shape == (m, inter)
+    ref = torch.nn.functional.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
+    torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=2e-2 * math.sqrt(k) / 4)
