@@ -102,6 +102,76 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_kernel(
   }
 }
 
+// Fast path for head sizes that are a multiple of 64 with half-split pairing and rotary_dim/2 a
+// multiple of 64 (D = 128 or 256 fully rotated): lane l holds elements l, l+64, ..., so both
+// members of every rotation pair sit in one lane: no LDS, no barrier.  One wave takes
+// `heads_per_wave` consecutive heads of one token.
+template <typename T, int E>
+__global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
+    T* __restrict__ qkv, const int* __restrict__ slot_mapping, const float* __restrict__ q_w,
+    const float* __restrict__ k_w, float eps, const float* __restrict__ cos_sin, int rotary_dim,
+    T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size, int nq, int nkv,
+    int heads_per_wave) {
+  constexpr int D = E * 64;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const long long t = blockIdx.x;
+  const int n_heads = nq + 2 * nkv;
+  T* row = qkv + t * (long long)n_heads * D;
+  const long long slot = slot_mapping ? (long long)slot_mapping[t] : -1;
+  const bool store = (slot >= 0) && (k_pages != nullptr);
+  const long long page = store ? slot / page_size : 0;
+  const int off = store ? (int)(slot - page * page_size) : 0;
+  const int half = rotary_dim / 2, HE = half / 64;   // pair (e, e + HE) for e < HE
+  float cs[E], sn[E];                                 // cos/sin of this lane's pair indices
+  if (cos_sin) {
+#pragma unroll
+    for (int e = 0; e < E; ++e)
+      if (e < HE) {
+        cs[e] = cos_sin[t * rotary_dim + e * 64 + lane];
+        sn[e] = cos_sin[t * rotary_dim + half + e * 64 + lane];
+      }
+  }
+  const int h0 = (blockIdx.y * 4 + wid) * heads_per_wave;
+  for (int head = h0; head < h0 + heads_per_wave && head < n_heads; ++head) {
+    T* x = row + (long long)head * D;
+    float v[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) v[e] = to_f32(x[e * 64 + lane]);
+    if (head >= nq + nkv) {  // v head: copied to its (transposed) page
+      if (store) {
+        T* dst = v_pages + (page * nkv + (head - nq - nkv)) * (long long)D * page_size + off;
+#pragma unroll
+        for (int e = 0; e < E; ++e) dst[(long long)(e * 64 + lane) * page_size] = from_f32<T>(v[e]);
+      }
+      continue;
+    }
+    const bool is_q = head < nq;
+    if (!is_q && !store) continue;
+    const float* w = is_q ? q_w : k_w;
+    if (w) {
+      float ss = 0.f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) ss += v[e] * v[e];
+      ss = wave_sum(ss);
+      const float inv = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] = v[e] * inv * w[e * 64 + lane];
+    }
+    if (cos_sin) {
+#pragma unroll
+      for (int e = 0; e < E; ++e)
+        if (e < HE) {
+          const float a = v[e], b = v[e + HE];
+          v[e] = a * cs[e] - b * sn[e];
+          v[e + HE] = b * cs[e] + a * sn[e];
+        }
+    }
+    T* dst = is_q ? x : k_pages + ((page * nkv + (head - nq)) * page_size + off) * (long long)D;
+#pragma unroll
+    for (int e = 0; e < E; ++e) dst[e * 64 + lane] = from_f32<T>(v[e]);
+  }
+}
+
 #define DEFINE_ROPE(SUF, T)                                                                        \
   extern "C" int jv_qk_norm_rope_write_##SUF(                                                      \
       void* qkv, const int* slot_mapping, const float* q_w, const float* k_w, float eps,           \
@@ -111,6 +181,21 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_kernel(
     if (D > ROPE_MAX_D || rotary_dim > D || (rotary_dim & 1)) return (int)hipErrorInvalidValue;    \
     const int n_heads = nq + 2 * nkv;                                                              \
     if ((n_heads + 3) / 4 > 65535) return (int)hipErrorInvalidValue;                               \
+    const int half = rotary_dim / 2;                                                               \
+    if ((D == 128 || D == 256) && !interleaved && (!cos_sin || (half % 64 == 0 && half > 0))) {    \
+      /* many tokens: a wave walks several heads; few tokens: one head per wave for parallelism */ \
+      const int hpw = n_tokens >= 256 ? (n_heads + 3) / 4 : 1;                                     \
+      const int gy = (n_heads + 4 * hpw - 1) / (4 * hpw);                                          \
+      if (D == 128)                                                                                \
+        hipLaunchKernelGGL((qk_norm_rope_write_fast_kernel<T, 2>), dim3(n_tokens, gy), dim3(256),  \
+                           0, (hipStream_t)stream, (T*)qkv, slot_mapping, q_w, k_w, eps, cos_sin,  \
+                           rotary_dim, (T*)k_pages, (T*)v_pages, page_size, nq, nkv, hpw);         \
+      else                                                                                         \
+        hipLaunchKernelGGL((qk_norm_rope_write_fast_kernel<T, 4>), dim3(n_tokens, gy), dim3(256),  \
+                           0, (hipStream_t)stream, (T*)qkv, slot_mapping, q_w, k_w, eps, cos_sin,  \
+                           rotary_dim, (T*)k_pages, (T*)v_pages, page_size, nq, nkv, hpw);         \
+      return JV_LAUNCH_CHECK();                                                                    \
+    }                                                                                              \
     hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(n_tokens, (n_heads + 3) / 4), dim3(256), \
                        4 * D * sizeof(float), (hipStream_t)stream, (T*)qkv, slot_mapping, q_w,     \
                        k_w, eps, cos_sin, rotary_dim, interleaved, (T*)k_pages, (T*)v_pages,       \

@@ -127,15 +127,24 @@ def rope_reference(x, pos, inv_freq, rotary_dim, interleaved):
     return out
 
 
+ROPE_CASES = [(4, 2, 16, 16, False, True, 11), (5, 5, 48, 48, False, True, 11), (6, 2, 128, 128, False, True, 11),
+              (3, 1, 80, 32, False, False, 11), (4, 4, 32, 32, True, True, 11), (8, 2, 256, 64, True, False, 11),
+              (8, 2, 256, 256, False, True, 11), (4, 4, 256, 128, False, True, 11), (32, 8, 128, 128, False, True, 300),
+              (5, 1, 128, 128, False, False, 260), (2, 2, 64, 64, False, True, 270)]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nq,nkv,d,rotary_dim,interleaved,with_norm",
-                         [(4, 2, 16, 16, False, True), (5, 5, 48, 48, False, True), (6, 2, 128, 128, False, True),
-                          (3, 1, 80, 32, False, False), (4, 4, 32, 32, True, True), (8, 2, 256, 64, True, False)])
-def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_norm):
-    t, page_size, pages, eps = 11, 4, 9, 1e-5
+@pytest.mark.parametrize("nq,nkv,d,rotary_dim,interleaved,with_norm,t", ROPE_CASES)
+def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_norm, t):
+    page_size, eps = 4, 1e-5
+    pages = t + 2
     qkv = randn(t, (nq + 2 * nkv) * d, dtype=dtype, seed=11)
-    pos = torch.tensor([0, 1, 2, 3, 100, 101, 4095, 7, 8, 9, 31999], dtype=torch.int32).cuda()
-    slots = torch.tensor([4, 5, 6, 7, 32, 33, 12, -1, 20, 21, 35], dtype=torch.int32).cuda()
+    g = torch.Generator().manual_seed(t)
+    pos_list = ([0, 1, 2, 3, 100, 101, 4095, 7, 8, 9, 31999] + torch.randint(0, 200, (max(0, t - 11),), generator=g).tolist())[:t]
+    slot_list = (torch.randperm((pages - 1) * page_size, generator=g)[:t] + page_size).tolist()   # distinct, none in page 0
+    slot_list[7] = -1
+    pos = torch.tensor(pos_list, dtype=torch.int32).cuda()
+    slots = torch.tensor(slot_list, dtype=torch.int32).cuda()
     qw = (1 + 0.1 * randn(d, seed=12)) if with_norm else None
     kw = (1 + 0.1 * randn(d, seed=13)) if with_norm else None
     inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rotary_dim, 2, dtype=torch.float32) / rotary_dim))).cuda()
@@ -157,21 +166,21 @@ def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_nor
     # large positions: the angle itself carries float rounding (pos * inv_freq ~ 3e4 * 1 has ulp 2e-3)
     big = dict(rtol=1e-2, atol=1e-2) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
     small = tol(dtype, f32=2e-5, bf16=2e-2)
-    near = pos.cpu() < 200
-    torch.testing.assert_close(got_q[near.cuda()], q[near.cuda()], **small)
+    near = (pos.cpu() < 200).cuda()
+    torch.testing.assert_close(got_q[near], q[near], **small)
     torch.testing.assert_close(got_q, q, **big)
     exp_k = torch.zeros(pages, nkv, page_size, d).cuda()
     exp_v = torch.zeros(pages, nkv, d, page_size).cuda()     # values are stored transposed
-    for i, s in enumerate(slots.tolist()):
-        if s >= 0:
-            exp_k[s // page_size, :, s % page_size] = k[i]
-            exp_v[s // page_size, :, :, s % page_size] = v[i]
+    for i, s_ in enumerate(slot_list):
+        if s_ >= 0:
+            exp_k[s_ // page_size, :, s_ % page_size] = k[i]
+            exp_v[s_ // page_size, :, :, s_ % page_size] = v[i]
     torch.testing.assert_close(k_pages.float(), exp_k, **big)
     torch.testing.assert_close(v_pages.float(), exp_v, rtol=0, atol=0)  # values are copied untouched
-    written = torch.zeros(pages * page_size, dtype=torch.bool)
-    written[[s for s in slots.tolist() if s >= 0]] = True
-    untouched = ~written.view(pages, page_size).cuda()
-    assert (k_pages.float().abs().sum((1, 3))[untouched] == 0).all()  # nothing beside the named slots
+    # without pages nothing is stored and q is still prepared (a run that reads another's cache)
+    qkv2 = x.reshape(t, -1).to(dtype).contiguous()
+    K().qk_norm_rope_write(qkv2, None, qw, kw, eps, table, rotary_dim, interleaved, None, None, page_size, nq, nkv, d)
+    torch.testing.assert_close(qkv2.float().view(t, nq + 2 * nkv, d)[:, :nq], got_q, rtol=0, atol=0)
 
 
 # ------------------------------------------------------------------ paged attention
