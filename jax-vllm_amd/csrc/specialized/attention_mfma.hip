@@ -25,6 +25,7 @@
 //                   partial (max, sum, acc) are merged in LDS; with num_splits > 1 several
 //                   blocks share a request's keys and a second kernel merges their partials.
 #include "../common.h"
+#include <type_traits>
 
 #ifndef JV_HEAD_DIM
 #error "compile with -DJV_HEAD_DIM=<head size>"
@@ -36,7 +37,8 @@ constexpr int NDT = D / 16;                // 16-wide tiles of the head dimensio
 constexpr int DK = (D + 31) / 32 * 32;     // head dimension padded to the QK contraction step
 constexpr int NKS = DK / 32;
 constexpr int BN = 64;                     // keys per LDS tile (prefill)
-constexpr int KS_STRIDE = DK + 8;          // bf16 elements per key row in LDS
+constexpr int KS_STRIDE = DK + 16;         // bf16 elements per key row in LDS: with a row stride of 8 dwords mod 16,
+                                           // 16-byte reads of 16 rows run at the full LDS rate (measured)
 constexpr int VT_STRIDE = BN + 8;          // bf16 elements per d row in LDS (rows 16-byte aligned, 4 banks apart)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -66,7 +68,7 @@ struct AttnArgs {
   int table_stride;
   const int* cu_seqlens;      // [requests + 1]
   const int* context_lens;    // [requests] keys stored before this step
-  const int* work;            // prefill: [n_work][2] = (request, first row of a block of 128); decode: [n_work] = request
+  const int* work;            // prefill: [n_work][3] = (request, first row of group 0, first row of group 1 or -1); decode: [n_work] = request
   int page_size, page_shift, nq, nkv;   // page_shift: log2(page_size) or -1
   float scale_log2;           // softmax scale * log2(e)
   int window;                 // <= 0: none
@@ -77,50 +79,64 @@ struct AttnArgs {
 };
 
 // ------------------------------------------------------------------------------------ prefill
-// 128 rows per block: 4 waves x 2 row tiles of 16 (one row tile, 64 rows, for head sizes above
-// 128).  Every K fragment and every V^T fragment read
-// from LDS feeds both row tiles of the wave.  The next tile's K/V are fetched from global memory
-// into registers while the current tile is multiplied, and written to LDS between two barriers.
-// Keys are masked only on tiles that cross a row's causal limit or window edge.
-constexpr int RT = D <= 128 ? 2 : 1;        // row tiles per wave (one for large heads: registers)
-constexpr int BM = 4 * RT * 16;            // rows per block
+// A block of 4 waves works on one or two GROUPS of 64 rows of one request and one kv head: wave w
+// takes rows 16w..16w+15 of each group (two groups for head sizes up to 128, one above: registers).
+// The host pairs a group that sees many keys with one that sees few, so that all blocks and all
+// waves have about the same number of (row tile, key tile) products; where both groups see a key
+// tile, every K fragment and V^T fragment read from LDS feeds both.  K/V tiles of 64 keys go
+// global -> registers while the previous tile is multiplied, and registers -> LDS between two
+// barriers.  Keys are masked only on tiles that cross a row's causal limit or window edge.
+constexpr int RT = D <= 128 ? 2 : 1;       // row groups per block = row tiles per wave
+constexpr int GROUP_ROWS = 64;             // 4 waves x 16 rows
 constexpr int KCH = BN * (DK / 8);         // 16-byte pieces of a K tile
 constexpr int VCH = D * (BN / 8);          // 16-byte pieces of a V^T tile
 constexpr int KPT = (KCH + 255) / 256;     // pieces per thread
 constexpr int VPT = (VCH + 255) / 256;
-constexpr int TBL_MAX = 2048;              // page-table entries a block keeps in LDS
+constexpr int TBL_MAX = 2048;              // page-table entries a block keeps in LDS at a time
+constexpr int NO_GAP = 0x7fffffff;
 
 #if JV_HEAD_DIM <= 128
 #define PREFILL_OCCUPANCY __attribute__((amdgpu_waves_per_eu(2, 2)))  // two waves per SIMD: one's softmax hides the other's MFMA
 #else
 #define PREFILL_OCCUPANCY
 #endif
+// PAGES: 1 = the page size is 8, 16, 32 or 64 (pages tile the 64 keys: a thread's slot in its
+// page is the same in every tile), 2 = a larger power of two, 0 = any other multiple of 8.
+template <int PAGES>
 __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(AttnArgs p) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[BN * KS_STRIDE];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[D * VT_STRIDE];
   __shared__ int page_ids[TBL_MAX];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, lc = lane >> 4;
-  const int r = p.work[2 * blockIdx.x], m0 = p.work[2 * blockIdx.x + 1];
-  const int g = blockIdx.y;
+  // consecutive blocks take the kv heads of one work item: with the heaviest items first the whole
+  // grid is heaviest-first, and (blocks going round the chip's 8 dies) a kv head's keys stay in
+  // the L2 of nkv/8 dies, or of one
+  const int g = blockIdx.x % p.nkv, item = blockIdx.x / p.nkv;
+  const int r = p.work[3 * item];
   const int G = p.nq / p.nkv, P = p.page_size;
-  const PageSplit ps{P, p.page_shift};
+  const PageSplit ps{P, PAGES == 0 ? -1 : p.page_shift};
   const int q_start = p.cu_seqlens[r], q_len = p.cu_seqlens[r + 1] - q_start;
   const int ctx = p.context_lens[r];
   const int M = q_len * G;
   const int* gtable = p.block_tables + (long long)r * p.table_stride;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  // this lane's rows: one per row tile
-  int row[RT], qi[RT], hg[RT], pos[RT];
+  // this lane's rows (one per group), and per group the key ranges of the block and of the wave
+  int qi[RT], hg[RT], pos[RT];
   bool row_ok[RT];
   bf16x8 qf[RT][NKS];
+  int blk_begin[RT], blk_end[RT];          // keys [begin, end) some row of the block's group sees; empty if no group
+  bool wave_live[RT];
+  int wave_kv_begin[RT], wave_kv_end[RT];  // keys some row of the wave's tile sees
+  int wave_full_begin[RT], wave_min_pos[RT];  // keys in [full_begin, min_pos] are seen by every row of the tile
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
-    row[t] = m0 + (wave * RT + t) * 16 + li;
-    row_ok[t] = row[t] < M;
-    qi[t] = row_ok[t] ? row[t] / G : 0;
-    hg[t] = row_ok[t] ? row[t] - qi[t] * G : 0;
+    const int m0 = p.work[3 * item + 1 + t];       // first row of the group, or -1
+    const int row = m0 + wave * 16 + li;
+    row_ok[t] = m0 >= 0 && row < M;
+    qi[t] = row_ok[t] ? row / G : 0;
+    hg[t] = row_ok[t] ? row - qi[t] * G : 0;
     pos[t] = ctx + qi[t];
     const bf16_t* qrow = p.q + (long long)(q_start + qi[t]) * p.q_row_stride + (long long)(g * G + hg[t]) * D;
 #pragma unroll
@@ -128,40 +144,58 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
       const int d0 = ks * 32 + lc * 8;
       qf[t][ks] = (row_ok[t] && d0 < D) ? *(const bf16x8*)(qrow + d0) : zero8;
     }
+    blk_begin[t] = blk_end[t] = 0;
+    if (m0 >= 0 && m0 < M) {
+      const int last_row = (M < m0 + GROUP_ROWS ? M : m0 + GROUP_ROWS) - 1;
+      blk_end[t] = ctx + last_row / G + 1;
+      if (p.window > 0) {
+        blk_begin[t] = ctx + m0 / G - p.window + 1;
+        if (blk_begin[t] < 0) blk_begin[t] = 0;
+      }
+    }
+    const int wave_first = m0 + wave * 16;
+    wave_live[t] = m0 >= 0 && wave_first < M;
+    const int wave_last = (M < wave_first + 16 ? M : wave_first + 16) - 1;
+    wave_kv_end[t] = wave_live[t] ? ctx + wave_last / G + 1 : 0;
+    wave_min_pos[t] = ctx + wave_first / G;
+    wave_kv_begin[t] = wave_full_begin[t] = 0;
+    if (p.window > 0 && wave_live[t]) {
+      wave_kv_begin[t] = wave_min_pos[t] - p.window + 1;
+      if (wave_kv_begin[t] < 0) wave_kv_begin[t] = 0;
+      wave_full_begin[t] = ctx + wave_last / G - p.window + 1;
+      if (wave_full_begin[t] < 0) wave_full_begin[t] = 0;
+    }
   }
-  // key range of the block and of this wave (rows of a wave are contiguous: 32 of them)
-  const int last_row = (M < m0 + BM ? M : m0 + BM) - 1;
-  const int kv_end = ctx + last_row / G + 1;
-  int kv_begin = 0;
-  if (p.window > 0) {
-    kv_begin = ctx + m0 / G - p.window + 1;
-    if (kv_begin < 0) kv_begin = 0;
+  // The tiles the block walks: those of the one range, or of the union of the two; when a window
+  // leaves a gap between them the walk jumps from gap_from to gap_to (both multiples of BN).
+  int j_first, kv_end, gap_from = NO_GAP, gap_to = NO_GAP;
+  {
+    int b0 = blk_begin[0] / BN * BN, e0 = blk_end[0];
+    int b1 = b0, e1 = 0;
+    if (RT > 1) { b1 = blk_begin[RT - 1] / BN * BN; e1 = blk_end[RT - 1]; }
+    if (e1 <= b1) { b1 = b0; e1 = e0; }             // no second group
+    if (e0 <= b0) { b0 = b1; e0 = e1; }             // no first group
+    if (b1 < b0) { int x = b0; b0 = b1; b1 = x; x = e0; e0 = e1; e1 = x; }
+    j_first = b0;
+    kv_end = e0 > e1 ? e0 : e1;
+    const int e0_up = (e0 + BN - 1) / BN * BN;
+    if (b1 > e0_up) { gap_from = e0_up; gap_to = b1; }
   }
-  const int wave_first = m0 + wave * RT * 16;
-  const int wave_last = (M < wave_first + RT * 16 ? M : wave_first + RT * 16) - 1;
-  const bool wave_live = wave_first < M;
-  const int wave_kv_end = wave_live ? ctx + wave_last / G + 1 : 0;     // keys >= this are invisible to all rows
-  const int wave_min_pos = ctx + wave_first / G;                       // keys <= this are visible to all rows
-  int wave_kv_begin = 0, wave_full_begin = 0;                          // window: first visible key of any / of all rows
-  if (p.window > 0 && wave_live) {
-    wave_kv_begin = wave_min_pos - p.window + 1;
-    if (wave_kv_begin < 0) wave_kv_begin = 0;
-    wave_full_begin = ctx + wave_last / G - p.window + 1;
-    if (wave_full_begin < 0) wave_full_begin = 0;
-  }
+  auto next_tile = [&](int j0) { return j0 + BN == gap_from ? gap_to : j0 + BN; };
+  if (kv_end <= j_first) return;                    // nothing to do (the same in every thread)
 
-  // the block's slice of the request's page table goes to LDS once: a tile's loads then hang
-  // on one global access, not on two in a row
-  // (from the first key of the first TILE, which may lie before kv_begin, to the last key read)
-  const int j_first = kv_begin / BN * BN;
-  const int first_page = ps.index(j_first);
-  const int n_pages = ps.index(kv_end + P - 1) - first_page;
-  const bool table_in_lds = n_pages <= TBL_MAX;
-  if (table_in_lds)
-    for (int i = tid; i < n_pages; i += 256) page_ids[i] = gtable[first_page + i];
-  auto page_of = [&](int j) -> long long {
-    return table_in_lds ? page_ids[ps.index(j) - first_page] : gtable[ps.index(j)];
+  // A slice of the request's page table sits in LDS: a tile's loads then hang on one global
+  // access, not on two in a row.  It starts at the page of the first key of the first tile and
+  // is moved forward when a tile reaches past its end.
+  const int last_page = ps.index(kv_end - 1);
+  int seg_first = 0;
+  auto load_table = [&](int j) {        // called by all threads, between barriers
+    seg_first = ps.index(j);
+    int n = last_page - seg_first + 1;
+    if (n > TBL_MAX) n = TBL_MAX;
+    for (int i = tid; i < n; i += 256) page_ids[i] = gtable[seg_first + i];
   };
+  load_table(j_first);
   __syncthreads();
 
   float m_run[RT], l_lane[RT];
@@ -174,13 +208,11 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
     for (int dt = 0; dt < NDT; ++dt) acc[t][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // piece c of a V^T tile -> (d, 8-key chunk).  When pages tile the 64 keys (page size 8, 16, 32
-  // or 64) consecutive threads walk one page's [D][P] block, which is contiguous in memory;
-  // otherwise chunk-major order.
-  const bool pages_tile = ps.shift >= 3 && ps.shift <= 6;
-  const int cpp_shift = ps.shift - 3;                  // log2(chunks per page row)
+  // piece c of a V^T tile -> (d, 8-key chunk).  When pages tile the 64 keys consecutive threads
+  // walk one page's [D][P] block, which is contiguous in memory; otherwise chunk-major order.
+  const int cpp_shift = ps.shift - 3;                  // PAGES == 1: log2(chunks per page row)
   auto v_piece = [&](int c, int& d, int& kc) {
-    if (pages_tile) {
+    if (PAGES == 1) {
       const int q = c >> cpp_shift;                    // (page in tile, d), D rows per page
       const int pg = q / D;
       d = q - pg * D;
@@ -190,142 +222,237 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
       kc = c - d * (BN / 8);
     }
   };
-  // ---- global -> registers for one tile; keys at or past kv_end become zeros
+  // ---- global -> registers for one tile.  Nothing here looks at a loaded value or branches per
+  // lane, so the loads stay in flight while the previous tile is multiplied.  A piece past the
+  // last key reads the same slot of the last page (allocated memory, masked later by position),
+  // and what must be zero is made zero when the registers are written to LDS.
+  const unsigned page_stride = (unsigned)p.nkv * (unsigned)P * (unsigned)D;   // elements; the host checks it fits
+  // per-thread constants of the pieces: the element offset inside a page; a piece's first key in
+  // the tile is recomputed where it is needed (registers are scarce here)
+  auto k_piece_key = [&](int i) {
+    int c = tid + i * 256;
+    if (KCH % 256 != 0 && c > KCH - 1) c = KCH - 1;
+    return c / (DK / 8);
+  };
+  auto v_piece_key = [&](int i) {
+    int c = tid + i * 256;
+    if (VCH % 256 != 0 && c > VCH - 1) c = VCH - 1;
+    int d, kc;
+    v_piece(c, d, kc);
+    return kc * 8;
+  };
+  int k_off[KPT], v_off[VPT];
+#pragma unroll
+  for (int i = 0; i < KPT; ++i) {
+    int c = tid + i * 256;
+    if (KCH % 256 != 0 && c > KCH - 1) c = KCH - 1;
+    const int key = c / (DK / 8);
+    int dc = c - key * (DK / 8);
+    if (DK != D && dc * 8 >= D) dc = 0;
+    k_off[i] = (g * P + (PAGES == 1 ? (key & (P - 1)) : 0)) * D + dc * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    int c = tid + i * 256;
+    if (VCH % 256 != 0 && c > VCH - 1) c = VCH - 1;
+    int d, kc;
+    v_piece(c, d, kc);
+    v_off[i] = (g * D + d) * P + (PAGES == 1 ? ((kc * 8) & (P - 1)) : 0);
+  }
   bf16x8 kreg[KPT], vreg[VPT];
   auto fetch = [&](int j0) {
+    int j_hi = j0 + BN - 1;
+    if (j_hi > kv_end - 1) j_hi = kv_end - 1;
+    if (ps.index(j_hi) - seg_first >= TBL_MAX) {   // same decision in every thread
+      __syncthreads();
+      load_table(j0);
+      __syncthreads();
+    }
+    const int tile_page = ps.index(j0) - seg_first, end_page = last_page - seg_first;
+#pragma unroll
+    for (int i = 0; i < KPT; ++i) {
+      int pi, off = k_off[i];
+      if (PAGES == 1) {
+        pi = tile_page + (k_piece_key(i) >> ps.shift);
+      } else {
+        const int j = j0 + k_piece_key(i);
+        pi = ps.index(j) - seg_first;
+        off += ps.slot(j) * D;
+      }
+      if (pi > end_page) pi = end_page;
+      const unsigned page = (unsigned)page_ids[pi];
+      kreg[i] = *(const bf16x8*)(p.k_pages + ((unsigned long long)page * page_stride + (unsigned)off));
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      int pi, off = v_off[i];
+      if (PAGES == 1) {
+        pi = tile_page + (v_piece_key(i) >> ps.shift);
+      } else {
+        const int j = j0 + v_piece_key(i);
+        pi = ps.index(j) - seg_first;
+        off += ps.slot(j);
+      }
+      if (pi > end_page) pi = end_page;
+      const unsigned page = (unsigned)page_ids[pi];
+      vreg[i] = *(const bf16x8*)(p.v_pages + ((unsigned long long)page * page_stride + (unsigned)off));
+    }
+  };
+  // ---- registers -> LDS.  K columns that pad the head size and V entries of keys at or past
+  // kv_end become zeros (their probabilities are zeros, and zero times a stale NaN is not).
+  auto stage = [&](int j0) {
 #pragma unroll
     for (int i = 0; i < KPT; ++i) {
       const int c = tid + i * 256;
       const int key = c / (DK / 8), dc = c - key * (DK / 8);
-      const int j = j0 + key;
-      bf16x8 v = zero8;
-      if (c < KCH && j < kv_end && dc * 8 < D) {
-        const long long page = page_of(j);
-        v = *(const bf16x8*)(p.k_pages + ((page * p.nkv + g) * P + ps.slot(j)) * (long long)D + dc * 8);
-      }
-      kreg[i] = v;
+      bf16x8 v = kreg[i];
+      if (DK != D && dc * 8 >= D) v = zero8;
+      if (KCH % 256 == 0 || c < KCH) *(bf16x8*)(Ks + key * KS_STRIDE + dc * 8) = v;
     }
+    const bool last_tile = j0 + BN > kv_end;      // the same in every thread
 #pragma unroll
     for (int i = 0; i < VPT; ++i) {
       const int c = tid + i * 256;
       int d, kc;
       v_piece(c, d, kc);
-      const int j = j0 + kc * 8;
-      bf16x8 v = zero8;
-      if (c < VCH && j < kv_end) {
-        const long long page = page_of(j);
-        v = *(const bf16x8*)(p.v_pages + ((page * p.nkv + g) * D + d) * (long long)P + ps.slot(j));
-        if (j + 8 > kv_end) {
+      bf16x8 v = vreg[i];
+      if (last_tile) {
+        const int j = j0 + kc * 8;
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (j + e >= kv_end) v[e] = (bf16_t)0.f;
-        }
+        for (int e = 0; e < 8; ++e)
+          if (j + e >= kv_end) v[e] = (bf16_t)0.f;
       }
-      vreg[i] = v;
-    }
-  };
-  auto stage = [&]() {
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-      const int c = tid + i * 256;
-      const int key = c / (DK / 8), dc = c - key * (DK / 8);
-      if (c < KCH) *(bf16x8*)(Ks + key * KS_STRIDE + dc * 8) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-      const int c = tid + i * 256;
-      int d, kc;
-      v_piece(c, d, kc);
-      if (c < VCH) *(bf16x8*)(Vt + d * VT_STRIDE + kc * 8) = vreg[i];
+      if (VCH % 256 == 0 || c < VCH) *(bf16x8*)(Vt + d * VT_STRIDE + kc * 8) = v;
     }
   };
 
-  if (j_first < kv_end) fetch(j_first);
-  for (int j0 = j_first; j0 < kv_end; j0 += BN) {
-    __syncthreads();          // everyone is done with the previous tile in LDS
-    stage();
-    __syncthreads();
-    if (j0 + BN < kv_end) fetch(j0 + BN);   // in flight while this tile is multiplied
-
-    if (wave_live && j0 < wave_kv_end && j0 + BN > wave_kv_begin) {
-      f32x4 s[RT][4];
+  // ---- one key tile times the row tiles named by MASK (bit t: the wave's tile of group t).
+  // LDS fragments are read one group ahead of the products that use them (K: the 4 key tiles of one
+  // 32-wide slice of the head; V^T: 2 head tiles of one 32-key half); the scheduling fences keep
+  // the compiler from moving a group's reads down to their first use, where every product would
+  // wait a full LDS round trip.
+  constexpr int VG = 2;                                  // head tiles per V^T fragment group
+  constexpr int GPK = (NDT + VG - 1) / VG;               // groups per 32-key half
+  auto read_k = [&](bf16x8 (&f)[4], int ks) {
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
+    for (int kt = 0; kt < 4; ++kt) f[kt] = *(const bf16x8*)(Ks + (kt * 16 + li) * KS_STRIDE + ks * 32 + lc * 8);
+  };
+  auto read_v = [&](bf16x8 (&f)[VG], int q) {
+    const int kk = q / GPK, d0 = (q - kk * GPK) * VG;
 #pragma unroll
-        for (int t = 0; t < RT; ++t) s[t][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-          const bf16x8 a = *(const bf16x8*)(Ks + (kt * 16 + li) * KS_STRIDE + ks * 32 + lc * 8);
-#pragma unroll
-          for (int t = 0; t < RT; ++t) s[t][kt] = mfma16(a, qf[t][ks], s[t][kt]);
-        }
+    for (int i = 0; i < VG; ++i) {
+      if (d0 + i < NDT) {
+        const bf16_t* vrow = Vt + ((d0 + i) * 16 + li) * VT_STRIDE + lc * 4;
+        const bf16x4 a0 = *(const bf16x4*)(vrow + (2 * kk) * 16);
+        const bf16x4 a1 = *(const bf16x4*)(vrow + (2 * kk + 1) * 16);
+        f[i] = bf16x8{a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
       }
-      // interior tile: every key visible to every row of the wave -> no per-element mask
-      const bool interior = (j0 + BN - 1 <= wave_min_pos) && (p.window <= 0 || j0 >= wave_full_begin);
+    }
+  };
+  auto multiply = [&](auto mask_const, int j0) {
+    constexpr int MASK = decltype(mask_const)::value;
+    f32x4 s[RT][4];
 #pragma unroll
-      for (int t = 0; t < RT; ++t) {
-        float tmax = -INFINITY;
-        if (interior) {
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
-          for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < 4; ++kt) s[t][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    bf16x8 kf[2][4];
+    read_k(kf[0], 0);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float v = s[t][kt][e] * p.scale_log2;
-              s[t][kt][e] = v;
-              tmax = fmaxf(tmax, v);
-            }
-        } else {
+    for (int ks = 0; ks < NKS; ++ks) {
+      if (ks + 1 < NKS) read_k(kf[(ks + 1) & 1], ks + 1);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int j = j0 + kt * 16 + lc * 4 + e;
-              const bool ok = row_ok[t] && j <= pos[t] && (p.window <= 0 || j > pos[t] - p.window);
-              const float v = ok ? s[t][kt][e] * p.scale_log2 : -INFINITY;
-              s[t][kt][e] = v;
-              tmax = fmaxf(tmax, v);
-            }
-        }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run[t], tmax);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run[t] - m_use);
-        float psum = 0.f;
+        for (int t = 0; t < RT; ++t)
+          if ((MASK >> t) & 1) s[t][kt] = mfma16(kf[ks & 1][kt], qf[t][ks], s[t][kt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    bf16x8 vf[2][VG];
+    read_v(vf[0], 0);                    // on its way during the softmax
+    __builtin_amdgcn_sched_barrier(0);
+    bf16x8 pb[2][RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) {
+      if (!((MASK >> t) & 1)) continue;
+      // interior tile: every key visible to every row of the tile -> no per-element mask
+      const bool interior = (j0 + BN - 1 <= wave_min_pos[t]) && (p.window <= 0 || j0 >= wave_full_begin[t]);
+      float tmax = -INFINITY;
+      // the maximum is taken over raw scores (the scale is positive); the scale enters in the
+      // exponent's multiply-add: p = exp2(s * scale_log2 - m * scale_log2)
+      if (interior) {
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) tmax = fmaxf(tmax, s[t][kt][e]);
+      } else {
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const float pv = fast_exp2(s[t][kt][e] - m_use);
-            s[t][kt][e] = pv;
-            psum += pv;
+            const int j = j0 + kt * 16 + lc * 4 + e;
+            const bool ok = row_ok[t] && j <= pos[t] && (p.window <= 0 || j > pos[t] - p.window);
+            const float v = ok ? s[t][kt][e] : -INFINITY;
+            s[t][kt][e] = v;
+            tmax = fmaxf(tmax, v);
           }
-        l_lane[t] = l_lane[t] * alpha + psum;
-        m_run[t] = m_new;
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) acc[t][dt] *= alpha;
       }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run[t], tmax);                       // raw-score units
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
+      const float alpha = fast_exp2(m_run[t] * p.scale_log2 - m_use);  // exp2(-inf) = 0 on the first tile
+      float psum = 0.f;
 #pragma unroll
-      for (int kk = 0; kk < 2; ++kk) {
-        bf16x8 b[RT];
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float pv = fast_exp2(fmaf(s[t][kt][e], p.scale_log2, -m_use));
+          s[t][kt][e] = pv;
+          psum += pv;
+        }
+      l_lane[t] = l_lane[t] * alpha + psum;
+      m_run[t] = m_new;
+#pragma unroll
+      for (int dt = 0; dt < NDT; ++dt) acc[t][dt] *= alpha;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          pb[kk][t][e] = (bf16_t)s[t][2 * kk][e];
+          pb[kk][t][4 + e] = (bf16_t)s[t][2 * kk + 1][e];
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < 2 * GPK; ++q) {
+      if (q + 1 < 2 * GPK) read_v(vf[(q + 1) & 1], q + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      const int kk = q / GPK, d0 = (q - kk * GPK) * VG;
+#pragma unroll
+      for (int i = 0; i < VG; ++i)
 #pragma unroll
         for (int t = 0; t < RT; ++t)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            b[t][e] = (bf16_t)s[t][2 * kk][e];
-            b[t][4 + e] = (bf16_t)s[t][2 * kk + 1][e];
-          }
-#pragma unroll
-        for (int dt = 0; dt < NDT; ++dt) {
-          const bf16_t* vrow = Vt + (dt * 16 + li) * VT_STRIDE + lc * 4;
-          const bf16x4 a0 = *(const bf16x4*)(vrow + (2 * kk) * 16);
-          const bf16x4 a1 = *(const bf16x4*)(vrow + (2 * kk + 1) * 16);
-          const bf16x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-#pragma unroll
-          for (int t = 0; t < RT; ++t) acc[t][dt] = mfma16(a, b[t], acc[t][dt]);
-        }
-      }
+          if (d0 + i < NDT && ((MASK >> t) & 1)) acc[t][d0 + i] = mfma16(vf[q & 1][i], pb[kk][t], acc[t][d0 + i]);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  };
+
+  fetch(j_first);
+  for (int j0 = j_first; j0 < kv_end;) {
+    const int j_next = next_tile(j0);
+    stage(j0);
+    __syncthreads();
+    if (j_next < kv_end) fetch(j_next);        // in flight while this tile is multiplied
+    int mask = 0;
+#pragma unroll
+    for (int t = 0; t < RT; ++t)
+      if (wave_live[t] && j0 < wave_kv_end[t] && j0 + BN > wave_kv_begin[t]) mask |= 1 << t;
+    if (RT > 1 && mask == 3) multiply(std::integral_constant<int, 3>{}, j0);
+    else if (RT > 1 && mask == 2) multiply(std::integral_constant<int, 2>{}, j0);
+    else if (mask == 1) multiply(std::integral_constant<int, 1>{}, j0);
+    __syncthreads();
+    j0 = j_next;
   }
 
 #pragma unroll
@@ -346,7 +473,9 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
   }
 }
 
-extern "C" int jv_attn_prefill_rows_per_block() { return BM; }
+// the host's plan: rows per group, and groups a work item may name
+extern "C" int jv_attn_prefill_group_rows() { return GROUP_ROWS; }
+extern "C" int jv_attn_prefill_groups_per_item() { return RT; }
 
 // ------------------------------------------------------------------------------------ decode
 constexpr int BND = 32;  // keys per wave iteration
@@ -566,8 +695,11 @@ extern "C" int jv_attn_prefill(void* out, const void* q, long long q_row_stride,
   a.page_size = page_size; a.nq = nq; a.nkv = nkv;
   a.scale_log2 = scale * 1.4426950408889634f; a.window = window; a.num_splits = 1;
   if (int e = check_common(a)) return e;
-  if (nkv > 65535) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_work, nkv), dim3(256), 0, (hipStream_t)stream, a);
+  if ((long long)nkv * page_size * D >= (1ll << 31)) return (int)hipErrorInvalidValue;   // offsets inside a page are 32-bit
+  if ((long long)n_work * nkv >= (1ll << 31)) return (int)hipErrorInvalidValue;
+  const int mode = (a.page_shift >= 3 && a.page_shift <= 6) ? 1 : (a.page_shift > 6 ? 2 : 0);
+  void (*kernel)(AttnArgs) = mode == 1 ? attn_prefill_kernel<1> : (mode == 2 ? attn_prefill_kernel<2> : attn_prefill_kernel<0>);
+  hipLaunchKernelGGL(kernel, dim3(n_work * nkv), dim3(256), 0, (hipStream_t)stream, a);
   return JV_LAUNCH_CHECK();
 }
 

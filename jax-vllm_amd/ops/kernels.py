@@ -333,9 +333,10 @@ def sample(logits: torch.Tensor, temperature=None, keys=None, out=None) -> torch
 MFMA_ATTENTION_MAX_HEAD_DIM = 256
 
 
-def attn_prefill_rows(head_dim: int) -> int:
-    """Rows (query, head-in-group pairs) of one block of the prefill kernel."""
-    return 128 if head_dim <= 128 else 64
+def attn_prefill_geometry(head_dim: int) -> tuple[int, int]:
+    """(rows of a group, groups a work item of the prefill kernel may name).  A row is a (query,
+    head-in-group) pair; a block's 4 waves take 16 rows each of every group of its item."""
+    return 64, (2 if head_dim <= 128 else 1)
 
 
 def mfma_attention_supported(dtype, head_dim: int, page_size: int) -> bool:
@@ -367,12 +368,13 @@ def _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlen
 
 def attn_prefill_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, n_work,
                       nq, nkv, head_dim, scale, window=0) -> None:
-    """Causal attention of prompt portions.  ``work`` is int32 [n_work, 2]: (request index, first row)
-    for every block of ``attn_prefill_rows(head_dim)`` rows, a row being a (query, head-in-group) pair of one
-    kv head."""
+    """Causal attention of prompt portions.  ``work`` is int32 [n_work, 3]: (request index, first row
+    of a group, first row of a second group of the same request or -1), see ``attn_prefill_geometry``;
+    every row of every request must be in exactly one group.  Pairing a group that sees many keys with
+    one that sees few gives all blocks the same amount of work."""
     page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
                              nq, nkv, head_dim)
-    _need(work.numel() >= 2 * n_work, "work list shorter than n_work")
+    _need(work.numel() >= 3 * n_work, "work list shorter than n_work")
     lib = library.attention(head_dim)
     _check(
         lib.jv_attn_prefill(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages),

@@ -2,10 +2,12 @@
 
 bfloat16 with a head size and page size the matrix-core kernels are built for: requests with
 one token in the step go to the decode kernel (keys shared out to several blocks when few
-requests would leave the chip idle), all others to the prefill kernel in blocks of 128 (or 64)
-(query, head-in-group) rows, heaviest blocks first.  Everything else (float32, other head
-sizes) runs the generic float-math kernel.  The plan depends on the step's lengths and on
-the heads-per-group ratio only, so it is built once per step and shared by all layers.
+requests would leave the chip idle), all others to the prefill kernel in groups of 64 (query,
+head-in-group) rows; a work item pairs a group that sees many keys with one of the same request
+that sees few, so that all blocks carry the same load, heaviest items first.  Everything else
+(float32, other head sizes) runs the generic float-math kernel.  The plan depends on the
+step's lengths, the heads-per-group ratio and whether the layer has a window, so it is built
+once per step and shared by all layers alike.
 """
 from __future__ import annotations
 
@@ -18,11 +20,12 @@ from ..ops import kernels as K
 
 TARGET_BLOCKS = 512          # about two blocks per compute unit
 MIN_KEYS_PER_SPLIT = 128     # one 32-key tile for each of a block's 4 waves
+BALANCE_BLOCKS = 768         # up to here prefill work items pair light row groups with heavy ones
 
 
 @dataclass
 class MfmaPlan:
-    prefill_work: Optional[torch.Tensor]   # int32 [n, 2]
+    prefill_work: Optional[torch.Tensor]   # int32 [n, 3]
     n_prefill: int
     decode_work: Optional[torch.Tensor]    # int32 [n]
     n_decode: int
@@ -37,29 +40,65 @@ def decode_splits(n_decode: int, blocks_per_request: int, max_kv_len: int) -> in
     return max(1, min(by_fill, by_len))
 
 
-def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, device) -> MfmaPlan:
-    g = nq // nkv
-    rows_per_block = K.attn_prefill_rows(head_dim)
-    prefill, decode = [], []
-    max_kv_decode = 1
-    for r, (ql, cl) in enumerate(zip(ctx.q_lens_host, ctx.context_lens_host)):
-        if ql == 1:
-            decode.append(r)
-            max_kv_decode = max(max_kv_decode, cl + 1)
+KEY_TILE = 64                # keys of one tile of the prefill kernel
+
+
+def prefill_work_items(q_lens, context_lens, g: int, window: int, group_rows: int, groups_per_item: int,
+                       balance: bool = True):
+    """Work items (request, first row of group 0, first row of group 1 or -1) of the prefill kernel
+    for the requests with more than one token, heaviest first.  Rows are (query, head-in-group)
+    pairs.  With ``balance`` and no window the i-th lightest group of a request is paired with its
+    i-th heaviest: every pair then walks about the same number of (row tile, key tile) products,
+    which matters when the items are so few that the heaviest one decides the time.  Otherwise
+    neighbours are paired: they share nearly all their keys, so every fragment read feeds both."""
+    items = []
+    for r, (ql, cl) in enumerate(zip(q_lens, context_lens)):
+        if ql <= 1:
+            continue
+        groups = []
+        for m0 in range(0, ql * g, group_rows):
+            last_row = min(ql * g, m0 + group_rows) - 1
+            end = cl + last_row // g + 1
+            begin = max(0, cl + m0 // g - window + 1) if window else 0
+            groups.append((-(-end // KEY_TILE) - begin // KEY_TILE, m0))
+        if groups_per_item < 2:
+            items.extend((t, r, m0, -1) for t, m0 in groups)
+        elif window or not balance:
+            for i in range(0, len(groups) - 1, 2):
+                items.append((groups[i][0] + groups[i + 1][0], r, groups[i][1], groups[i + 1][1]))
+            if len(groups) % 2:
+                items.append((groups[-1][0], r, groups[-1][1], -1))
         else:
-            for m0 in range(0, ql * g, rows_per_block):
-                last_row = min(ql * g, m0 + rows_per_block) - 1
-                prefill.append((cl + last_row // g + 1, r, m0))
-    prefill.sort(key=lambda w: -w[0])
+            lo, hi = 0, len(groups) - 1          # groups are in ascending order of keys seen
+            while lo < hi:
+                items.append((groups[lo][0] + groups[hi][0], r, groups[hi][1], groups[lo][1]))
+                lo, hi = lo + 1, hi - 1
+            if lo == hi:
+                items.append((groups[lo][0], r, groups[lo][1], -1))
+    items.sort(key=lambda w: -w[0])
+    return [(r, a, b) for _, r, a, b in items]
+
+
+def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> MfmaPlan:
+    g = nq // nkv
+    group_rows, groups_per_item = K.attn_prefill_geometry(head_dim)
+    # measured on 32 q heads, 8 kv heads of 128: balancing wins while the blocks fit on the chip about
+    # one and a half times (2,048 tokens: 87 against 102 us), sharing wins beyond (8,192: 887 against 1,036)
+    rows = sum(ql * g for ql in ctx.q_lens_host if ql > 1)
+    blocks = -(-rows // (group_rows * groups_per_item)) * nkv
+    prefill = prefill_work_items(ctx.q_lens_host, ctx.context_lens_host, g, window, group_rows, groups_per_item,
+                                 balance=blocks <= BALANCE_BLOCKS)
+    decode = [r for r, ql in enumerate(ctx.q_lens_host) if ql == 1]
+    max_kv_decode = max([ctx.context_lens_host[r] + 1 for r in decode], default=1)
     splits = decode_splits(len(decode), nkv * (-(-g // 16)), max_kv_decode) if decode else 1
-    flat = [x for _, r, m0 in prefill for x in (r, m0)] + decode
+    flat = [x for item in prefill for x in item] + decode
     dev = torch.tensor(flat, dtype=torch.int32).pin_memory().to(device, non_blocking=True) if flat else None
     n_pre = len(prefill)
     scratch = None
     if decode and splits > 1:
         scratch = torch.empty(K.attn_decode_scratch_floats(len(decode), nq, splits, head_dim),
                               dtype=torch.float32, device=device)
-    return MfmaPlan(dev[: 2 * n_pre] if n_pre else None, n_pre, dev[2 * n_pre:] if decode else None, len(decode),
+    return MfmaPlan(dev[: 3 * n_pre] if n_pre else None, n_pre, dev[3 * n_pre:] if decode else None, len(decode),
                     splits, scratch)
 
 
@@ -71,10 +110,10 @@ def run(att, out, qkv, ctx, mem) -> None:
             ctx.positions, att.nq, att.nkv, att.d, att.scale, att.window or 0,
         )
         return
-    key = ("mfma_attention_plan", att.nq, att.nkv, att.d)
+    key = ("mfma_attention_plan", att.nq, att.nkv, att.d, bool(att.window))
     plan = ctx.plans.get(key)
     if plan is None:
-        plan = ctx.plans[key] = plan_mfma(ctx, att.nq, att.nkv, att.d, qkv.device)
+        plan = ctx.plans[key] = plan_mfma(ctx, att.nq, att.nkv, att.d, att.window or 0, qkv.device)
     tables = ctx.block_tables[mem.group]
     if plan.n_prefill:
         K.attn_prefill_mfma(out, qkv, q_row_stride, mem.k_pages, mem.v_pages, tables, ctx.cu_seqlens,

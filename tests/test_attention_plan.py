@@ -1,0 +1,54 @@
+"""The host-side plan of the prefill attention kernel: which rows go to which block."""
+import random
+
+from jax_vllm_amd.parts.attention_backend import KEY_TILE, decode_splits, prefill_work_items
+
+
+def _tiles(cl, m0, ql, g, rows, window):
+    last_row = min(ql * g, m0 + rows) - 1
+    end = cl + last_row // g + 1
+    begin = max(0, cl + m0 // g - window + 1) if window else 0
+    return -(-end // KEY_TILE) - begin // KEY_TILE
+
+
+def test_every_row_is_in_exactly_one_group():
+    rng = random.Random(0)
+    for _ in range(200):
+        g = rng.choice([1, 2, 4, 5, 20])
+        window = rng.choice([0, 0, 7, 100])
+        per_item = rng.choice([1, 2])
+        q_lens = [rng.choice([1, 2, 3, 17, 64, 65, 300]) for _ in range(rng.randint(1, 4))]
+        ctx = [rng.choice([0, 1, 63, 64, 1000]) for _ in q_lens]
+        items = prefill_work_items(q_lens, ctx, g, window, 64, per_item)
+        seen = sorted((r, m0) for r, a, b in items for m0 in (a, b) if m0 >= 0)
+        want = sorted((r, m0) for r, ql in enumerate(q_lens) if ql > 1 for m0 in range(0, ql * g, 64))
+        assert seen == want
+        assert all(a >= 0 for _, a, _ in items)
+        if per_item == 1:
+            assert all(b == -1 for _, _, b in items)
+
+
+def test_single_token_requests_are_left_to_the_decode_kernel():
+    assert prefill_work_items([1, 1], [5, 9], 4, 0, 64, 2) == []
+
+
+def test_pairs_balance_the_load_and_heaviest_come_first():
+    ql, g = 2048, 4
+    items = prefill_work_items([ql], [0], g, 0, 64, 2)
+    loads = [sum(_tiles(0, m0, ql, g, 64, 0) for m0 in (a, b) if m0 >= 0) for _, a, b in items]
+    assert loads == sorted(loads, reverse=True)
+    assert max(loads) - min(loads) <= 1                      # unpaired, the spread would be 31
+    assert len(items) == ql * g // 128
+
+
+def test_window_pairs_neighbours():
+    items = prefill_work_items([512], [0], 1, 64, 64, 2)
+    assert sorted((a, b) for _, a, b in items) == [(m0, m0 + 64) for m0 in range(0, 512, 128)]
+    items = prefill_work_items([512], [0], 1, 0, 64, 2, balance=False)
+    assert [(a, b) for _, a, b in items] == [(m0, m0 + 64) for m0 in range(384, -1, -128)]   # heaviest first
+
+
+def test_decode_splits_fill_the_chip_but_keep_a_tile_per_wave():
+    assert decode_splits(1, 8, 100) == 1                     # too few keys to share out
+    assert decode_splits(1, 8, 8192) == 64
+    assert decode_splits(64, 8, 8192) == 1                   # enough blocks already

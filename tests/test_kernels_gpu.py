@@ -355,22 +355,51 @@ MFMA_PREFILL_CASES = [c for c in ATT_CASES if c[3] % 8 == 0] + [
     (4, 4, 112, 24, [(30, 40), (0, 3)], None),
     (8, 1, 64, 8, [(5, 70)], 17),
     (40, 2, 32, 16, [(10, 9)], None),      # 20 heads per group: rows of one query span two 16-row tiles
+    (8, 2, 128, 16, [(0, 700)], None),     # 44 groups: light ones paired with heavy ones
+    (8, 2, 64, 16, [(100, 300)], 50),      # window: paired groups far apart leave a gap of key tiles between them
+    (4, 1, 128, 32, [(64, 129), (0, 64)], 40),
+    (2, 1, 16, 8, [(17000, 40)], None),    # more pages than the kernel keeps of the table at a time
+    (2, 1, 16, 8, [(17000, 200)], 100),
 ]
 
 
+def _prefill_work(reqs, g, d, window, plan):
+    """Work items of the prefill kernel: by the engine's planner, one group per item, or every group
+    in the item's second place."""
+    from jax_vllm_amd.parts.attention_backend import prefill_work_items
+
+    group_rows, per_item = K().attn_prefill_geometry(d)
+    singles = [(r, m0) for r, (c, ql) in enumerate(reqs) for m0 in range(0, ql * g, group_rows)]
+    if plan == "planner":
+        items = prefill_work_items([ql for _, ql in reqs], [c for c, _ in reqs], g, window or 0, group_rows, per_item)
+        items += [(r, 0, -1) for r, (c, ql) in enumerate(reqs) if ql == 1]      # the planner leaves these to decode
+    elif plan == "second" and per_item > 1:
+        items = [(r, -1, m0) for r, m0 in singles]
+    elif plan == "far" and per_item > 1:         # first with last, window or not
+        items = []
+        for r in range(len(reqs)):
+            mine = [m0 for rr, m0 in singles if rr == r]
+            while len(mine) > 1:
+                items.append((r, mine.pop(0), mine.pop(-1)))
+            items += [(r, m0, -1) for m0 in mine]
+    else:
+        items = [(r, m0, -1) for r, m0 in singles]
+    covered = sorted((r, m0) for r, a, b in items for m0 in (a, b) if m0 >= 0)
+    assert covered == sorted(singles)
+    return torch.tensor([x for it in items for x in it], dtype=torch.int32).cuda(), len(items)
+
+
+@pytest.mark.parametrize("plan", ["planner", "single", "second", "far"])
 @pytest.mark.parametrize("case", MFMA_PREFILL_CASES,
                          ids=[f"h{c[0]}g{c[1]}d{c[2]}p{c[3]}w{c[5]}n{len(c[4])}" for c in MFMA_PREFILL_CASES])
-def test_mfma_prefill_attention(case):
+def test_mfma_prefill_attention(case, plan):
     nq, nkv, d, page_size, reqs, window = case
     scale = 1.0 / math.sqrt(d)
     qs, ks, vs, dev = _mfma_inputs(nq, nkv, d, page_size, reqs)
-    g = nq // nkv
-    rpb = K().attn_prefill_rows(d)
-    work = [x for r, (c, ql) in enumerate(reqs) for m0 in range(0, ql * g, rpb) for x in (r, m0)]
+    work, n_work = _prefill_work(reqs, nq // nkv, d, window, plan)
     out = torch.full((dev["n"], nq * d), float("nan"), dtype=torch.bfloat16).cuda()
     K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
-                          dev["ctx"], torch.tensor(work, dtype=torch.int32).cuda(), len(work) // 2, nq, nkv, d,
-                          scale, window or 0)
+                          dev["ctx"], work, n_work, nq, nkv, d, scale, window or 0)
     ref = _mfma_reference(qs, ks, vs, reqs, scale, window, nq, d)
     torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
 
@@ -426,7 +455,7 @@ def test_mfma_attention_finds_one_far_key(kernel, far_key):
             torch.tensor([0, 1], dtype=torch.int32).cuda(), torch.tensor([ctx - 1], dtype=torch.int32).cuda())
     scale = 1.0 / math.sqrt(d)
     if kernel == "prefill":
-        K().attn_prefill_mfma(*args, torch.tensor([0, 0], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
+        K().attn_prefill_mfma(*args, torch.tensor([0, 0, -1], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
     else:
         splits = int(kernel[-1])
         scratch = torch.empty(max(1, K().attn_decode_scratch_floats(1, nq, splits, d))).cuda()
@@ -450,7 +479,7 @@ def test_mfma_attention_ignores_garbage_past_the_context():
     ref = _mfma_reference(qs, ks, vs, reqs, scale, None, nq, d)
     out = torch.zeros(dev["n"], nq * d, dtype=torch.bfloat16).cuda()
     K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
-                          dev["ctx"], torch.tensor([0, 0], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
+                          dev["ctx"], torch.tensor([0, 0, -1], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
     K().attn_decode_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
                          dev["ctx"], torch.tensor([1], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale)
     torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
@@ -468,7 +497,7 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     out = torch.zeros(dev["n"], nq * d, dtype=torch.bfloat16).cuda()
     with pytest.raises(KernelArgumentError, match="multiple of 8"):
         K().attn_prefill_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
-                              dev["ctx"], torch.tensor([0, 0], dtype=torch.int32).cuda(), 1, nq, nkv, d, 0.1)
+                              dev["ctx"], torch.tensor([0, 0, -1], dtype=torch.int32).cuda(), 1, nq, nkv, d, 0.1)
 
 
 # ------------------------------------------------------------------ weight-streaming matrix product
