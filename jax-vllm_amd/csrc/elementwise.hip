@@ -84,8 +84,15 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restric
   const T* dr = delta ? delta + r * hidden : nullptr;
   T* o = out + i * hidden;
   const int nvec = hidden >> 2;
-  float4 x[ARN_MAX_V];
+  // every load (residual, delta, norm weight) is issued before the reduction: a short row's time is
+  // the sum of its dependent memory round trips, and the weights are cold in every layer
+  float4 x[ARN_MAX_V], ww[ARN_MAX_V];
   float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < ARN_MAX_V; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c < nvec) ww[k] = *(const float4*)(w + 4 * c);
+  }
 #pragma unroll
   for (int k = 0; k < ARN_MAX_V; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
@@ -106,9 +113,8 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restric
   for (int k = 0; k < ARN_MAX_V; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
     if (c < nvec) {
-      const float4 ww = *(const float4*)(w + 4 * c);
       const float4 v = x[k];
-      store4<T>(o + 4 * c, float4{v.x * inv * ww.x, v.y * inv * ww.y, v.z * inv * ww.z, v.w * inv * ww.w});
+      store4<T>(o + 4 * c, float4{v.x * inv * ww[k].x, v.y * inv * ww[k].y, v.z * inv * ww[k].z, v.w * inv * ww[k].w});
     }
   }
 }

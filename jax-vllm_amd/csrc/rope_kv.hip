@@ -134,9 +134,14 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
   const int h0 = (blockIdx.y * 4 + wid) * heads_per_wave;
   for (int head = h0; head < h0 + heads_per_wave && head < n_heads; ++head) {
     T* x = row + (long long)head * D;
-    float v[E];
+    float v[E], wv[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) v[e] = to_f32(x[e * 64 + lane]);
+    {  // the norm weights are asked for together with the head, not after its reduction
+      const float* w0 = head < nq ? q_w : (head < nq + nkv ? k_w : nullptr);
+#pragma unroll
+      for (int e = 0; e < E; ++e) wv[e] = w0 ? w0[e * 64 + lane] : 1.f;
+    }
     if (head >= nq + nkv) {  // v head: copied to its (transposed) page
       if (store) {
         T* dst = v_pages + (page * nkv + (head - nq - nkv)) * (long long)D * page_size + off;
@@ -155,7 +160,7 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
       ss = wave_sum(ss);
       const float inv = rsqrtf(ss / (float)D + eps);
 #pragma unroll
-      for (int e = 0; e < E; ++e) v[e] = v[e] * inv * w[e * 64 + lane];
+      for (int e = 0; e < E; ++e) v[e] = v[e] * inv * wv[e];
     }
     if (cos_sin) {
 #pragma unroll

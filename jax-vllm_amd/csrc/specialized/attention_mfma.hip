@@ -96,7 +96,7 @@ constexpr int TBL_MAX = 2048;              // page-table entries a block keeps i
 constexpr int NO_GAP = 0x7fffffff;
 
 #if JV_HEAD_DIM <= 128
-#define PREFILL_OCCUPANCY __attribute__((amdgpu_waves_per_eu(2, 2)))  // two waves per SIMD: one's softmax hides the other's MFMA
+#define PREFILL_OCCUPANCY __attribute__((amdgpu_waves_per_eu(2, 2)))  // two waves per SIMD (both kernels): one wave computes while the other waits
 #else
 #define PREFILL_OCCUPANCY
 #endif
@@ -480,7 +480,7 @@ extern "C" int jv_attn_prefill_groups_per_item() { return RT; }
 // ------------------------------------------------------------------------------------ decode
 constexpr int BND = 32;  // keys per wave iteration
 
-__global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs p) {
+__global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(AttnArgs p) {
   extern __shared__ float smem[];  // per wave: m[16], l[16], acc[16][D]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int li = lane & 15, lc = lane >> 4;
@@ -523,10 +523,13 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs p) {
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int t = t_lo + wave; t < t_hi; t += 4) {
+  // One tile's operands, global -> registers.  Nothing here looks at a loaded value, so a tile's
+  // loads are in flight while the tile before it is multiplied.  Keys at or past kv_len read the
+  // null page: their scores are masked by position, their V entries are zeroed before use.
+  //   K operand: lane (key li of sub-tile kt, chunk lc) <- 8 consecutive d of that key
+  //   V^T operand: lane (d = dt*16 + li, chunk lc) <- keys kt*16 + lc*4 .. +4 of that d
+  auto load_tile = [&](int t, bf16x8 (&kf)[2][NKS], bf16x4 (&vf)[2][NDT]) {
     const int j0 = t * BND;
-    // K operand: lane (key li of sub-tile kt, chunk lc) <- 8 consecutive d of that key
-    bf16x8 kf[2][NKS];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       const int j = j0 + kt * 16 + li;
@@ -536,13 +539,9 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs p) {
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         const int d0 = ks * 32 + lc * 8;
-        bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (ok && d0 < D) v = *(const bf16x8*)(krow + d0);
-        kf[kt][ks] = v;
+        kf[kt][ks] = *(const bf16x8*)(krow + (DK != D && d0 >= D ? 0 : d0));
       }
     }
-    // V^T operand: lane (d = dt*16 + li, chunk lc) <- keys kt*16 + lc*4 .. +4 of that d
-    bf16x4 vf[2][NDT];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       const int j = j0 + kt * 16 + lc * 4;
@@ -550,18 +549,26 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs p) {
       const long long page = ok ? table[ps.index(j)] : 0;
       const bf16_t* vbase = p.v_pages + (page * p.nkv + g) * (long long)D * P + (ok ? ps.slot(j) : 0);
 #pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        bf16x4 v = {0, 0, 0, 0};
-        if (ok) {
-          v = *(const bf16x4*)(vbase + (long long)(dt * 16 + li) * P);
-          if (j + 4 > kv_len) {
+      for (int dt = 0; dt < NDT; ++dt) vf[kt][dt] = *(const bf16x4*)(vbase + (long long)(dt * 16 + li) * P);
+    }
+  };
+  auto multiply = [&](int t, bf16x8 (&kf)[2][NKS], bf16x4 (&vf)[2][NDT]) {
+    const int j0 = t * BND;
+    if (DK != D) {                       // columns that pad the head size to the contraction step
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (j + e >= kv_len) v[e] = (bf16_t)0.f;
-          }
-        }
-        vf[kt][dt] = v;
-      }
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+          if (ks * 32 + lc * 8 >= D) kf[kt][ks] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+    if (j0 + BND > kv_len) {             // the last tile (the same in every lane): zero times a stale NaN is not zero
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (j0 + kt * 16 + lc * 4 + e >= kv_len) vf[kt][dt][e] = (bf16_t)0.f;
     }
     f32x4 s[2];
 #pragma unroll
@@ -603,6 +610,22 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs p) {
       const bf16x4 a0 = vf[0][dt], a1 = vf[1][dt];
       const bf16x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
       acc[dt] = mfma16(a, b, acc[dt] * alpha);
+    }
+  };
+  // two register sets take turns: while one tile is multiplied the wave's next one is on its way
+  {
+    bf16x8 kf_a[2][NKS], kf_b[2][NKS];
+    bf16x4 vf_a[2][NDT], vf_b[2][NDT];
+    int t = t_lo + wave;
+    if (t < t_hi) load_tile(t, kf_a, vf_a);
+    while (t < t_hi) {
+      if (t + 4 < t_hi) load_tile(t + 4, kf_b, vf_b);
+      multiply(t, kf_a, vf_a);
+      t += 4;
+      if (t >= t_hi) break;
+      if (t + 4 < t_hi) load_tile(t + 4, kf_a, vf_a);
+      multiply(t, kf_b, vf_b);
+      t += 4;
     }
   }
 
@@ -651,22 +674,42 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(AttnArgs p) {
 
 // merges the splits of one (request, head): grid (n_work, nq), D threads (rounded up to 64)
 __global__ void attn_decode_merge_kernel(AttnArgs p) {
-  const int w = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+  // All loads of a batch of 8 splits are issued before anything is computed from them: this
+  // kernel's time is its chain of dependent memory round trips, not its arithmetic.
+  const int w = blockIdx.x, head = blockIdx.y, d = threadIdx.x < D ? threadIdx.x : D - 1;
   const int r = p.work[w];
   const int tok = p.cu_seqlens[r];
   const long long base = ((long long)w * p.nq + head) * p.num_splits;
-  float mx = -INFINITY;
-  for (int s = 0; s < p.num_splits; ++s) mx = fmaxf(mx, p.part_ml[(base + s) * 2]);
-  if (d >= D) return;
-  float num = 0.f, den = 0.f;
-  for (int s = 0; s < p.num_splits; ++s) {
-    const float ms = p.part_ml[(base + s) * 2];
-    if (ms == -INFINITY) continue;
-    const float f = fast_exp2(ms - mx);
-    num += p.part_acc[(base + s) * D + d] * f;
-    den += p.part_ml[(base + s) * 2 + 1] * f;
+  const float2* ml = (const float2*)p.part_ml + base;      // (max, sum) per split
+  const float* pa = p.part_acc + base * D + d;
+  float mx = -INFINITY, num = 0.f, den = 0.f;
+  for (int s0 = 0; s0 < p.num_splits; s0 += 8) {
+    float2 v[8];
+    float a[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int s = s0 + i < p.num_splits ? s0 + i : p.num_splits - 1;   // a repeat, given no weight below
+      v[i] = ml[s];
+      a[i] = pa[(long long)s * D];
+    }
+    float bm = mx;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) bm = fmaxf(bm, v[i].x);
+    if (bm == -INFINITY) continue;                          // nothing stored in these splits or before
+    const float keep = fast_exp2(mx - bm);                  // 0 when mx is still -inf
+    num *= keep;
+    den *= keep;
+    mx = bm;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      // an empty split (max -inf) may hold anything in its accumulator: it gets no weight and is not read into the sum
+      const bool live = s0 + i < p.num_splits && v[i].x != -INFINITY;
+      const float f = live ? fast_exp2(v[i].x - mx) : 0.f;
+      num += live ? a[i] * f : 0.f;
+      den += live ? v[i].y * f : 0.f;
+    }
   }
-  p.out[(long long)tok * p.nq * D + (long long)head * D + d] = (bf16_t)(num / den);
+  if (threadIdx.x < D) p.out[(long long)tok * p.nq * D + (long long)head * D + d] = (bf16_t)(num / den);
 }
 
 // ------------------------------------------------------------------------------------ entry points
