@@ -72,6 +72,20 @@ __device__ __forceinline__ void store4(T* p, float4 v) {
 template <>
 __device__ __forceinline__ void store4<float>(float* p, float4 v) { *(float4*)p = v; }
 
+// eight neighbours as floats: one 16-byte load of bfloat16, two of float
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
+  typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+  const bf16x8_t x = *(const bf16x8_t*)p;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) v[e] = (float)x[e];
+}
+template <>
+__device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
 #define ARN_MAX_V 8
 template <typename T>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
@@ -144,20 +158,21 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* __restrict__ x,
 // out[t, j] = silu(gate) * up, silu(x) = x / (1 + exp(-x)), in float.  Two layouts of gu[t, 2*inter]:
 // halves (gate = gu[t, j], up = gu[t, inter + j]) or interleaved (gate = gu[t, 2j], up = gu[t, 2j+1]).
 // Interleaved layout (gate and up alternate along the row): out[t, j] = silu(gu[t, 2j]) * gu[t, 2j+1];
-// each thread takes two outputs (4 inputs) when inter is even.
+// each thread takes four outputs (8 inputs, 16 bytes of bfloat16) when inter % 4 == 0.
 template <typename T>
 __global__ void silu_mul_pairs_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
   const long long t = blockIdx.y;
-  const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 2;
+  const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (j >= inter) return;
   const T* gp = gu + t * 2 * inter + 2 * j;
   T* op = out + t * inter + j;
-  if (j + 1 < inter && (inter & 1) == 0) {
-    const float4 v = load4<T>(gp);
-    op[0] = from_f32<T>(v.x / (1.f + expf(-v.x)) * v.y);
-    op[1] = from_f32<T>(v.z / (1.f + expf(-v.z)) * v.w);
+  if ((inter & 3) == 0) {
+    float v[8];
+    load8<T>(gp, v);
+    store4<T>(op, float4{v[0] / (1.f + expf(-v[0])) * v[1], v[2] / (1.f + expf(-v[2])) * v[3],
+                         v[4] / (1.f + expf(-v[4])) * v[5], v[6] / (1.f + expf(-v[6])) * v[7]});
   } else {
-    for (int e = 0; e < 2 && j + e < inter; ++e) {
+    for (int e = 0; e < 4 && j + e < inter; ++e) {
       const float g = to_f32(gp[2 * e]), u = to_f32(gp[2 * e + 1]);
       op[e] = from_f32<T>(g / (1.f + expf(-g)) * u);
     }
@@ -232,7 +247,7 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
       T* o = (T*)out + t0 * inter;                                                                  \
       const T* g = (const T*)gu + t0 * 2 * inter;                                                   \
       if (interleaved) {                                                                            \
-        hipLaunchKernelGGL((silu_mul_pairs_kernel<T>), dim3(((inter + 1) / 2 + 255) / 256, ny),     \
+        hipLaunchKernelGGL((silu_mul_pairs_kernel<T>), dim3(((inter + 3) / 4 + 255) / 256, ny),     \
                            dim3(256), 0, (hipStream_t)stream, o, g, inter);                         \
       } else if (inter % 4 == 0) {                                                                         \
         hipLaunchKernelGGL((silu_mul_kernel<T, 4>), dim3((inter / 4 + 255) / 256, ny), dim3(256),   \
