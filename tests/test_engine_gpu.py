@@ -477,3 +477,158 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype):
     core.start_request("d")
     out = core.run([entry("d", reqs["c"])]).cpu().numpy()
     check_logits(dtype, out, plain(reqs["c"]), what="d after b")
+
+
+class TopOneExperts:
+    """A toy feed-forward with routing, defined and registered here: router logits in float, the
+    best expert of each token (lowest index on ties) runs a two-matrix ReLU feed-forward and its
+    output is scaled by the router's softmax weight of that expert."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int):
+        self.h, self.i, self.e = hidden_size, intermediate_size, num_experts
+
+    def tensors(self):
+        from jax_vllm_amd.parts import TensorSpec
+
+        t = {"router.weight": TensorSpec((self.e, self.h))}
+        for x in range(self.e):
+            t[f"experts.{x}.up.weight"] = TensorSpec((self.i, self.h))
+            t[f"experts.{x}.down.weight"] = TensorSpec((self.h, self.i))
+        return t
+
+    def bind(self, tensors, dtype):
+        self.t = tensors
+
+    def forward(self, x, ctx):
+        logits = x.float() @ self.t["router.weight"].float().t()
+        weight, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+        out = torch.zeros_like(x)
+        for e in range(self.e):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                hid = torch.relu(x[rows] @ self.t[f"experts.{e}.up.weight"].t())
+                out[rows] = ((hid @ self.t[f"experts.{e}.down.weight"].t()).float() * weight[rows, None]).to(x.dtype)
+        return out
+
+
+class LinearFrequencyRotation:
+    """A toy position encoding, defined and registered here: neighbouring pairs (2i, 2i+1) of the
+    first ``rotary_dim`` head elements turn by position * (i + 1) * step; the rest pass through."""
+
+    def __init__(self, rotary_dim: int, step: float):
+        self.rotary_dim, self.step = rotary_dim, step
+
+    def tensors(self):
+        return {}
+
+    def bind(self, tensors, dtype, device=None):
+        self.freq = (torch.arange(1, self.rotary_dim // 2 + 1, dtype=torch.float32) * self.step).to(device or "cuda")
+
+    def fused_arguments(self, ctx):
+        from jax_vllm_amd.ops import kernels as K
+
+        key = ("linear_frequency_table", self.rotary_dim, self.step)
+        if key not in ctx.extras:
+            ctx.extras[key] = K.rope_table(ctx.positions, self.freq)
+        return ctx.extras[key], self.rotary_dim, True
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_routed_feed_forward_and_toy_position_encoding(dtype):
+    """Layers pick their parts one by one: a routed feed-forward in one layer, a dense one in the
+    other, and attention with a position encoding of the test's own, all without a change to the
+    package.  The plain implementation is written out here."""
+    from jax_vllm_amd.config import register_architecture, resolve
+    from jax_vllm_amd.parts import DecoderModel, LayerRun, LayerSpec, ModelSpec, PartSpec, register_part
+    from jax_vllm_amd.weights.loader import TORCH_DTYPES, target_dtype
+
+    register_part("feed_forward", "top_one_experts", TopOneExperts)
+    register_part("position", "linear_frequency", LinearFrequencyRotation)
+    hidden, vocab, inter, heads, kvh, d, rot, step, eps = 40, 90, 56, 4, 2, 16, 8, 0.37, 1e-5
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": eps})
+    att = PartSpec("gqa_attention", dict(hidden_size=hidden, num_heads=heads, num_kv_heads=kvh, head_dim=d, qk_norm_eps=eps,
+                                         position=PartSpec("linear_frequency", {"rotary_dim": rot, "step": step})))
+    routed = PartSpec("top_one_experts", {"hidden_size": hidden, "intermediate_size": inter, "num_experts": 3})
+    dense = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter})
+
+    def build(_cfg):
+        return ModelSpec(
+            vocab_size=vocab, hidden_size=hidden,
+            embedding=PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": hidden}), embedding_prefix="emb.",
+            final_norm=norm, final_norm_prefix="norm.", head=PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": hidden}),
+            head_prefix="head.", tie_head_to_embedding=False,
+            layers=[LayerSpec(f"l{i}.", att, ff, PartSpec("prenorm", {"norm": norm}), "att.", "ff.")
+                    for i, ff in enumerate([routed, dense])],
+            schedule=[LayerRun(0), LayerRun(1)])
+
+    register_architecture("ToyRoutedModel", lambda c: c, build)
+    arch, cfg, _ = resolve({"architectures": ["ToyRoutedModel"]})
+    model = DecoderModel(arch.build_spec(cfg))
+    g = torch.Generator().manual_seed(21)
+    compute = TORCH_DTYPES[dtype]
+    w = {n: ((0.25 * torch.randn(ts.shape, generator=g)) if ts.role == "matrix" else 1 + 0.1 * torch.randn(ts.shape, generator=g))
+         .to(torch.bfloat16).float() for n, ts in model.tensor_specs().items()}
+    # the router separates its experts clearly, so that rounding does not flip a choice
+    w["l0.ff.router.weight"] = (w["l0.ff.router.weight"] * 6).to(torch.bfloat16).float()
+    model.bind({n: v.cuda().to(target_dtype(model.tensor_specs()[n].role, compute)) for n, v in w.items()}, compute)
+    core = make_core(None, dtype, 8, pages=30, seqs=2, model=model)
+
+    def rotate(x, pos):                      # x [heads, T, d]
+        ang = pos[:, None].float() * (torch.arange(1, rot // 2 + 1).float() * step)[None, :]
+        cos, sin = torch.cos(ang)[None], torch.sin(ang)[None]
+        a, b = x[..., 0:rot:2], x[..., 1:rot:2]
+        y = x.clone()
+        y[..., 0:rot:2] = a * cos - b * sin
+        y[..., 1:rot:2] = b * cos + a * sin
+        return y
+
+    def attention(p, x, pos):
+        t = x.shape[0]
+        q = (x @ w[f"{p}.q_proj.weight"].T).reshape(t, heads, d).transpose(0, 1)
+        k = (x @ w[f"{p}.k_proj.weight"].T).reshape(t, kvh, d).transpose(0, 1)
+        v = (x @ w[f"{p}.v_proj.weight"].T).reshape(t, kvh, d).transpose(0, 1)
+        q = rotate(P.rms_norm(w[f"{p}.q_norm.weight"], eps, q), pos)
+        k = rotate(P.rms_norm(w[f"{p}.k_norm.weight"], eps, k), pos)
+        o = P.attention_core(q, k, v, P.causal_mask(t, t)).transpose(0, 1).reshape(t, heads * d)
+        return o @ w[f"{p}.o_proj.weight"].T
+
+    def experts(p, x):
+        probs = torch.softmax(x @ w[f"{p}.router.weight"].T, dim=-1)
+        weight, choice = probs.max(dim=-1)
+        out = torch.zeros_like(x)
+        for t in range(x.shape[0]):
+            e = int(choice[t])
+            out[t] = (torch.relu(x[t] @ w[f"{p}.experts.{e}.up.weight"].T) @ w[f"{p}.experts.{e}.down.weight"].T) * weight[t]
+        return out, choice
+
+    def plain(tokens):
+        pos = torch.arange(len(tokens))
+        h = w["emb.weight"][torch.tensor(tokens)]
+        choices = None
+        for i in (0, 1):
+            h = h + attention(f"l{i}.att", P.rms_norm(w[f"l{i}.input_layernorm.weight"], eps, h), pos)
+            m = P.rms_norm(w[f"l{i}.post_attention_layernorm.weight"], eps, h)
+            if i == 0:
+                delta, choices = experts("l0.ff", m)
+            else:
+                delta = P.swiglu(w["l1.ff.gate_proj.weight"], w["l1.ff.up_proj.weight"], w["l1.ff.down_proj.weight"], m)
+            h = h + delta
+        return (P.rms_norm(w["norm.weight"], eps, h) @ w["head.weight"].T).numpy(), choices
+
+    rng = np.random.default_rng(8)
+    toks = rng.integers(0, vocab, size=70).tolist()
+    want, choices = plain(toks)
+    assert len(set(choices.tolist())) == 3                   # every expert is used
+    # a shift of all positions changes nothing where only distances count: the oracle's own check
+    # of its rotation (a wrong pairing or sign fails it)
+    x = torch.randn(heads, 5, d, generator=g)
+    s0 = torch.einsum("hqd,hkd->hqk", rotate(x, torch.arange(5)), rotate(x, torch.arange(5)))
+    s9 = torch.einsum("hqd,hkd->hqk", rotate(x, torch.arange(9, 14)), rotate(x, torch.arange(9, 14)))
+    torch.testing.assert_close(s0, s9, rtol=1e-4, atol=1e-4)
+    core.start_request("a")
+    got, at = [], 0
+    for n in [19, 2, 1, 30, 1, 1, 16]:
+        got.append(core.run([entry("a", toks[at:at + n])]).cpu().numpy())
+        at += n
+    assert at == len(toks)
+    check_logits(dtype, np.concatenate(got), want)

@@ -465,6 +465,67 @@ def test_mfma_attention_finds_one_far_key(kernel, far_key):
     torch.testing.assert_close(out.float().cpu(), expect, rtol=1e-2, atol=1e-2)
 
 
+def _loud_key_case(nq, nkv, d, ctx, ql, qi, key, seed):
+    """Random small q, k; query ``qi`` and key ``key`` get one large matching component, so that
+    the key decides the query's output if (and only if) the query may see it."""
+    g = torch.Generator().manual_seed(seed)
+    k = torch.randn(ctx + ql, nkv, d, generator=g) * 0.1
+    v = torch.randn(ctx + ql, nkv, d, generator=g)
+    q = torch.randn(ql, nq, d, generator=g) * 0.1
+    q[qi, :, 0] = 40.0
+    k[key, :, 0] = 40.0
+    bf = torch.bfloat16
+    return q.to(bf).float(), k.to(bf).float(), v.to(bf).float()
+
+
+EDGES = ["self", "future", "window_first", "before_window"]
+
+
+@pytest.mark.parametrize("kernel", ["generic", "prefill", "decode1", "decode3"])
+@pytest.mark.parametrize("edge", EDGES)
+def test_attention_edges_of_visibility(edge, kernel):
+    """A loud key is put exactly on, and exactly one beyond, the causal limit and the window's
+    first key of a query, for queries on both sides of the kernels' row and key tile borders.
+    An edge that is off by one gives the wrong key's value, not a small error."""
+    nq, nkv, d, page_size, window = 4, 2, 64, 16, 64
+    scale = 1.0 / math.sqrt(d)
+    bf = torch.bfloat16
+    decode = kernel.startswith("decode")
+    cases = [(c, 1, 0) for c in (70, 127, 128, 129, 200)] if decode else \
+        [(70, 70, qi) for qi in (0, 7, 8, 31, 32, 33, 68)]
+    for ctx, ql, qi in cases:
+        pos = ctx + qi
+        key = {"self": pos, "future": pos + 1, "window_first": pos - window + 1, "before_window": pos - window}[edge]
+        if key >= ctx + ql:
+            continue                                   # the last query has no future key in the cache
+        q, k, v = _loud_key_case(nq, nkv, d, ctx, ql, qi, key, seed=pos)
+        positions = torch.arange(ctx, ctx + ql)
+        ref = attention_reference(q, k, v, positions, scale, window).reshape(ql, nq * d)
+        visible = edge in ("self", "window_first")
+        if visible:                                    # the oracle itself must show the effect
+            torch.testing.assert_close(ref[qi].float().reshape(nq, d),
+                                       torch.repeat_interleave(v[key], nq // nkv, dim=0), rtol=1e-3, atol=1e-3)
+        k_pages, v_pages, tables = build_paged([k], [v], page_size, seed=pos)
+        out = torch.full((ql, nq * d), float("nan"), dtype=bf).cuda()
+        args = (out, q.reshape(ql, -1).to(bf).cuda(), nq * d, k_pages.to(bf).cuda(), v_pages.to(bf).cuda(),
+                tables.cuda())
+        cu = torch.tensor([0, ql], dtype=torch.int32).cuda()
+        cl = torch.tensor([ctx], dtype=torch.int32).cuda()
+        if kernel == "generic":
+            K().paged_attention_generic(*args, torch.zeros(ql, dtype=torch.int32).cuda(),
+                                        positions.to(torch.int32).cuda(), nq, nkv, d, scale, window)
+        elif kernel == "prefill":
+            work, n_work = _prefill_work([(ctx, ql)], nq // nkv, d, window, "single")
+            K().attn_prefill_mfma(*args, cu, cl, work, n_work, nq, nkv, d, scale, window)
+        else:
+            splits = int(kernel[-1])
+            scratch = torch.empty(max(1, K().attn_decode_scratch_floats(1, nq, splits, d))).cuda()
+            K().attn_decode_mfma(*args, cu, cl, torch.tensor([0], dtype=torch.int32).cuda(), 1, nq, nkv, d, scale,
+                                 window, splits, scratch)
+        torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2,
+                                   msg=lambda m: f"context {ctx}, query {qi}, key {key}: {m}")
+
+
 def test_mfma_attention_ignores_garbage_past_the_context():
     """Slots of the last page beyond the context hold NaN and infinity: they must not leak."""
     nq, nkv, d, page_size = 4, 2, 64, 16
