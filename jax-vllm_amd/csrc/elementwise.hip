@@ -87,6 +87,7 @@ __device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
 }
 
 #define ARN_MAX_V 8
+#define ARN_MAX_PARTS 4
 template <typename T>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
                                        const float* __restrict__ w, T* __restrict__ out,
@@ -117,6 +118,60 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restric
         v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
         if (!rows) *(float4*)(hr + 4 * c) = v;
       }
+      x[k] = v;
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+  for (int k = 0; k < ARN_MAX_V; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c < nvec) {
+      const float4 v = x[k];
+      store4<T>(o + 4 * c, float4{v.x * inv * ww[k].x, v.y * inv * ww[k].y, v.z * inv * ww[k].z, v.w * inv * ww[k].w});
+    }
+  }
+}
+
+// The same with the delta given as NP float partial products of a matrix product whose inner
+// size was shared out to NP blocks: parts[q][r][:], added first, in the order of q, then to the
+// residual.  Every load of the row is issued before anything is computed (the kernel's time is
+// its chain of memory round trips).
+template <typename T, int NP>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_parts_kernel(float* __restrict__ h, const float* __restrict__ parts, long long part_stride,
+                         const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
+                         int hidden, float eps) {
+  __shared__ float red[32];
+  const long long i = blockIdx.x;
+  const long long r = rows ? (long long)rows[i] : i;
+  float* hr = h + r * hidden;
+  const float* pr = parts + r * hidden;
+  T* o = out + i * hidden;
+  const int nvec = hidden >> 2;
+  float4 x[ARN_MAX_V], ww[ARN_MAX_V], e[ARN_MAX_V][NP];
+#pragma unroll
+  for (int k = 0; k < ARN_MAX_V; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c < nvec) {
+      ww[k] = *(const float4*)(w + 4 * c);
+      x[k] = *(const float4*)(hr + 4 * c);
+#pragma unroll
+      for (int q = 0; q < NP; ++q) e[k][q] = *(const float4*)(pr + q * part_stride + 4 * c);
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < ARN_MAX_V; ++k) {
+    const int c = threadIdx.x + k * blockDim.x;
+    if (c < nvec) {
+      float4 d = e[k][0];
+#pragma unroll
+      for (int q = 1; q < NP; ++q) { d.x += e[k][q].x; d.y += e[k][q].y; d.z += e[k][q].z; d.w += e[k][q].w; }
+      float4 v = x[k];
+      v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+      if (!rows) *(float4*)(hr + 4 * c) = v;
       x[k] = v;
       ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
@@ -227,6 +282,29 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
     } else {                                                                                        \
       hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(threads), 0, (hipStream_t)stream, \
                          h, (const T*)delta, w, (T*)out, rows, hidden, eps);                        \
+    }                                                                                               \
+    return JV_LAUNCH_CHECK();                                                                       \
+  }                                                                                                 \
+  /* the delta as n_parts float partial products [n_parts][rows of h][hidden], added in order */   \
+  extern "C" int jv_add_rmsnorm_parts_##SUF(float* h, const float* parts, int n_parts,              \
+                                            long long part_stride, const float* w, void* out,       \
+                                            const int* rows, int n_out, int hidden, float eps,      \
+                                            void* stream) {                                         \
+    if (n_out <= 0) return 0;                                                                       \
+    if (n_parts < 1 || n_parts > ARN_MAX_PARTS || hidden % 4 != 0 || hidden > 4 * ARN_MAX_V * 256)  \
+      return (int)hipErrorInvalidValue;                                                             \
+    const int nvec = hidden / 4;                                                                    \
+    const int vt = nvec >= 1024 ? 256 : (nvec >= 256 ? 128 : 64);                                   \
+    hipStream_t st = (hipStream_t)stream;                                                           \
+    switch (n_parts) {                                                                              \
+      case 1: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 1>), dim3(n_out), dim3(vt), 0, st, h, \
+                                 parts, part_stride, w, (T*)out, rows, hidden, eps); break;         \
+      case 2: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 2>), dim3(n_out), dim3(vt), 0, st, h, \
+                                 parts, part_stride, w, (T*)out, rows, hidden, eps); break;         \
+      case 3: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 3>), dim3(n_out), dim3(vt), 0, st, h, \
+                                 parts, part_stride, w, (T*)out, rows, hidden, eps); break;         \
+      default: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 4>), dim3(n_out), dim3(vt), 0, st,   \
+                                  h, parts, part_stride, w, (T*)out, rows, hidden, eps); break;     \
     }                                                                                               \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \

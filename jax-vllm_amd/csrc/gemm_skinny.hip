@@ -148,10 +148,15 @@ gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
 // into LDS (MP = 8 or 16 rows; B-operand lanes of rows >= MP read row % MP, their results are
 // never stored), one barrier, and the products run as the weights arrive.  One or two barriers
 // per phase instead of one per 128 columns.
+// K may also be shared out to gridDim.y blocks (k_per columns each, a multiple of KP): block
+// (tile, s) then writes the partial product of its columns to y + s * y_part, and whoever reads
+// y adds the parts in the order of s.  A narrow matrix gets enough blocks that way to keep the
+// memory system busy (a fifth of the chip's bandwidth is lost at 256 blocks against 1,024).
 template <int NL, typename OutT>
 __global__ void __launch_bounds__(1024)
 gemm_skinny_resident_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
-                            int M, int N, int K, long long ldx, long long ldy, int WK, int MP, int KP) {
+                            int M, int N, int K_all, long long ldx, long long ldy, int WK, int MP, int KP,
+                            int k_per, long long y_part) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16_t* xs = (bf16_t*)smem;                // [MP][KP + SK_PAD]
   const int LROW = KP + SK_PAD;
@@ -159,7 +164,11 @@ gemm_skinny_resident_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, 
   const int wk = tid >> 6, lane = tid & 63, li = lane & 15, lc = lane >> 4;
   const int n = blockIdx.x * 16 + li;
   const bool n_ok = n < N;
-  const bf16_t* wrow = W + (long long)(n_ok ? n : 0) * K + lc * 8;
+  const int kb = blockIdx.y * k_per;         // this block's columns are [kb, kb + K)
+  const int K = K_all - kb < k_per ? K_all - kb : k_per;
+  const bf16_t* wrow = W + (long long)(n_ok ? n : 0) * K_all + kb + lc * 8;
+  x += kb;
+  y += blockIdx.y * y_part;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   const int SL = NL * 32;                    // columns of one wave per phase; KP == WK * SL
   const int n_phase = (K + KP - 1) / KP;
@@ -212,9 +221,14 @@ gemm_skinny_resident_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, 
 
 template <int NL, typename OutT>
 static int launch_resident(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                           long long ldy, int WK, hipStream_t stream) {
+                           long long ldy, int WK, int ksplit, hipStream_t stream) {
   const int MP = M <= 8 ? 8 : 16;
   const int KP = WK * NL * 32;
+  // columns per block: the phases shared out evenly, whole phases each
+  const int phases = (K + KP - 1) / KP;
+  if (ksplit < 1 || ksplit > phases || ksplit > 65535) return (int)hipErrorInvalidValue;
+  const int k_per = (phases + ksplit - 1) / ksplit * KP;
+  if ((long long)k_per * (ksplit - 1) >= K) return (int)hipErrorInvalidValue;   // a block without columns
   size_t shmem = (size_t)MP * (KP + SK_PAD) * 2;
   if (shmem < (size_t)WK * 256 * 4) shmem = (size_t)WK * 256 * 4;
   if (shmem > 160 * 1024) return (int)hipErrorInvalidValue;
@@ -227,18 +241,20 @@ static int launch_resident(void* y, const void* x, const void* W, int M, int N, 
       raised = true;
     }
   }
-  hipLaunchKernelGGL((gemm_skinny_resident_kernel<NL, OutT>), dim3((N + 15) / 16), dim3(WK * 64), shmem, stream,
-                     (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, WK, MP, KP);
+  hipLaunchKernelGGL((gemm_skinny_resident_kernel<NL, OutT>), dim3((N + 15) / 16, ksplit), dim3(WK * 64), shmem,
+                     stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, WK, MP, KP, k_per,
+                     (long long)M * ldy);
   return JV_LAUNCH_CHECK();
 }
 
 template <typename OutT>
 static int dispatch_resident(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                             long long ldy, int WK, hipStream_t s) {
+                             long long ldy, int WK, int ksplit, hipStream_t s) {
   switch (nl) {
-    case 4: return launch_resident<4, OutT>(y, x, W, M, N, K, ldx, ldy, WK, s);
-    case 8: return launch_resident<8, OutT>(y, x, W, M, N, K, ldx, ldy, WK, s);
-    case 16: return launch_resident<16, OutT>(y, x, W, M, N, K, ldx, ldy, WK, s);
+    case 2: return launch_resident<2, OutT>(y, x, W, M, N, K, ldx, ldy, WK, ksplit, s);
+    case 4: return launch_resident<4, OutT>(y, x, W, M, N, K, ldx, ldy, WK, ksplit, s);
+    case 8: return launch_resident<8, OutT>(y, x, W, M, N, K, ldx, ldy, WK, ksplit, s);
+    case 16: return launch_resident<16, OutT>(y, x, W, M, N, K, ldx, ldy, WK, ksplit, s);
   }
   return (int)hipErrorInvalidValue;
 }
@@ -313,25 +329,28 @@ static void skinny_config(int M, int N, int K, int* wr, int* wk, int* nks) {
 //      silu(x.W[2j]) * (x.W[2j+1]) is bf16 [M, N/2] (the feed-forward's first product with its
 //      activation as epilogue).
 // wr, wk, nks: block shape (row tiles, K slices, MFMA steps per iteration); 0 picks them.
-// wr == -1 selects the resident-x organisation (M <= 16, no silu): wk waves, nks in {4, 8, 16}
+// wr == -1 selects the resident-x organisation (M <= 16, no silu): wk waves, nks in {2, 4, 8, 16}
 // weight pieces per wave and phase.
+// ksplit > 1 (resident-x organisation, float output only): K is shared out to ksplit blocks per
+// row tile and y is [ksplit][M][ldy], partial products that the reader adds in that order.
 extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
                                    long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
-                                   int wk, int nks, void* stream) {
+                                   int wk, int nks, int ksplit, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
   if (silu_pairs && (out_f32 || N % 2 != 0 || wr == -1)) return (int)hipErrorInvalidValue;
+  if (ksplit < 1 || (ksplit > 1 && (wr != -1 || !out_f32))) return (int)hipErrorInvalidValue;
   if (wr == -1) {
     if (M > 16 || wk < 1 || wk > 16) return (int)hipErrorInvalidValue;
     hipStream_t s = (hipStream_t)stream;
-    return out_f32 ? dispatch_resident<float>(nks, y, x, W, M, N, K, ldx, ldy, wk, s)
-                   : dispatch_resident<bf16_t>(nks, y, x, W, M, N, K, ldx, ldy, wk, s);
+    return out_f32 ? dispatch_resident<float>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s)
+                   : dispatch_resident<bf16_t>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s);
   }
   if (wr == 0 && wk == 0 && nks == 0 && M <= 2 && !silu_pairs && K >= 2048 && K <= 4096 && N >= 8192) {
     // one or two rows against a wide matrix: the resident-x organisation measured ~10 % faster
     hipStream_t s = (hipStream_t)stream;
-    return out_f32 ? dispatch_resident<float>(16, y, x, W, M, N, K, ldx, ldy, 8, s)
-                   : dispatch_resident<bf16_t>(16, y, x, W, M, N, K, ldx, ldy, 8, s);
+    return out_f32 ? dispatch_resident<float>(16, y, x, W, M, N, K, ldx, ldy, 8, 1, s)
+                   : dispatch_resident<bf16_t>(16, y, x, W, M, N, K, ldx, ldy, 8, 1, s);
   }
   int cwr, cwk, cnks;
   skinny_config(M, N, K, &cwr, &cwk, &cnks);

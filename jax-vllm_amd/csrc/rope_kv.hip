@@ -106,9 +106,10 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_kernel(
 // multiple of 64 (D = 128 or 256 fully rotated): lane l holds elements l, l+64, ..., so both
 // members of every rotation pair sit in one lane: no LDS, no barrier.  One wave takes
 // `heads_per_wave` consecutive heads of one token.
-template <typename T, int E>
+template <typename T, int E, int NP>
 __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
-    T* __restrict__ qkv, const int* __restrict__ slot_mapping, const float* __restrict__ q_w,
+    T* __restrict__ qkv, const float* __restrict__ parts, long long part_stride,
+    const int* __restrict__ slot_mapping, const float* __restrict__ q_w,
     const float* __restrict__ k_w, float eps, const float* __restrict__ cos_sin, int rotary_dim,
     T* __restrict__ k_pages, T* __restrict__ v_pages, int page_size, int nq, int nkv,
     int heads_per_wave) {
@@ -135,8 +136,25 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
   for (int head = h0; head < h0 + heads_per_wave && head < n_heads; ++head) {
     T* x = row + (long long)head * D;
     float v[E], wv[E];
+    if (NP == 0) {
 #pragma unroll
-    for (int e = 0; e < E; ++e) v[e] = to_f32(x[e * 64 + lane]);
+      for (int e = 0; e < E; ++e) v[e] = to_f32(x[e * 64 + lane]);
+    } else {
+      // the projection comes as NP float partial products [NP][tokens][heads * D] of a matrix
+      // product whose inner size was shared out: all are asked for at once and added in order
+      const float* px = parts + (t * n_heads + head) * (long long)D + lane;
+      float pv[NP > 0 ? NP : 1][E];
+#pragma unroll
+      for (int q = 0; q < NP; ++q)
+#pragma unroll
+        for (int e = 0; e < E; ++e) pv[q][e] = px[q * part_stride + e * 64];
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        v[e] = pv[0][e];
+#pragma unroll
+        for (int q = 1; q < NP; ++q) v[e] += pv[q][e];
+      }
+    }
     {  // the norm weights are asked for together with the head, not after its reduction
       const float* w0 = head < nq ? q_w : (head < nq + nkv ? k_w : nullptr);
 #pragma unroll
@@ -192,13 +210,15 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
       const int hpw = n_tokens >= 256 ? (n_heads + 3) / 4 : 1;                                     \
       const int gy = (n_heads + 4 * hpw - 1) / (4 * hpw);                                          \
       if (D == 128)                                                                                \
-        hipLaunchKernelGGL((qk_norm_rope_write_fast_kernel<T, 2>), dim3(n_tokens, gy), dim3(256),  \
-                           0, (hipStream_t)stream, (T*)qkv, slot_mapping, q_w, k_w, eps, cos_sin,  \
-                           rotary_dim, (T*)k_pages, (T*)v_pages, page_size, nq, nkv, hpw);         \
+        hipLaunchKernelGGL((qk_norm_rope_write_fast_kernel<T, 2, 0>), dim3(n_tokens, gy),          \
+                           dim3(256), 0, (hipStream_t)stream, (T*)qkv, (const float*)nullptr, 0ll, \
+                           slot_mapping, q_w, k_w, eps, cos_sin, rotary_dim, (T*)k_pages,          \
+                           (T*)v_pages, page_size, nq, nkv, hpw);                                  \
       else                                                                                         \
-        hipLaunchKernelGGL((qk_norm_rope_write_fast_kernel<T, 4>), dim3(n_tokens, gy), dim3(256),  \
-                           0, (hipStream_t)stream, (T*)qkv, slot_mapping, q_w, k_w, eps, cos_sin,  \
-                           rotary_dim, (T*)k_pages, (T*)v_pages, page_size, nq, nkv, hpw);         \
+        hipLaunchKernelGGL((qk_norm_rope_write_fast_kernel<T, 4, 0>), dim3(n_tokens, gy),          \
+                           dim3(256), 0, (hipStream_t)stream, (T*)qkv, (const float*)nullptr, 0ll, \
+                           slot_mapping, q_w, k_w, eps, cos_sin, rotary_dim, (T*)k_pages,          \
+                           (T*)v_pages, page_size, nq, nkv, hpw);                                  \
       return JV_LAUNCH_CHECK();                                                                    \
     }                                                                                              \
     hipLaunchKernelGGL(qk_norm_rope_write_kernel<T>, dim3(n_tokens, (n_heads + 3) / 4), dim3(256), \
@@ -210,3 +230,40 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
 
 DEFINE_ROPE(bf16, bf16_t)
 DEFINE_ROPE(f32, float)
+
+// The same with the projection given as n_parts (2..4) float partial products
+// [n_parts][tokens][heads * D]; q is written to `qkv` (the q heads of each row), k and v to their
+// pages.  Only what the fast path takes: head size 128 or 256, half-split pairing, fully rotated
+// or not rotated; anything else is refused (the caller then asks for a whole product).
+template <typename T, int E, int NP>
+static int launch_rope_parts(void* qkv, const float* parts, long long part_stride, const int* slot_mapping,
+                             const float* q_w, const float* k_w, float eps, const float* cos_sin, int rotary_dim,
+                             void* k_pages, void* v_pages, int page_size, int n_tokens, int nq, int nkv,
+                             void* stream) {
+  const int n_heads = nq + 2 * nkv;
+  const int hpw = n_tokens >= 256 ? (n_heads + 3) / 4 : 1;
+  const int gy = (n_heads + 4 * hpw - 1) / (4 * hpw);
+  hipLaunchKernelGGL((qk_norm_rope_write_fast_kernel<T, E, NP>), dim3(n_tokens, gy), dim3(256), 0,
+                     (hipStream_t)stream, (T*)qkv, parts, part_stride, slot_mapping, q_w, k_w, eps, cos_sin,
+                     rotary_dim, (T*)k_pages, (T*)v_pages, page_size, nq, nkv, hpw);
+  return JV_LAUNCH_CHECK();
+}
+
+extern "C" int jv_qk_norm_rope_write_parts_bf16(
+    void* qkv, const float* parts, int n_parts, long long part_stride, const int* slot_mapping, const float* q_w,
+    const float* k_w, float eps, const float* cos_sin, int rotary_dim, void* k_pages, void* v_pages,
+    int page_size, int n_tokens, int nq, int nkv, int D, void* stream) {
+  if (n_tokens <= 0) return 0;
+  const int half = rotary_dim / 2;
+  if ((D != 128 && D != 256) || n_parts < 2 || n_parts > 4 || (rotary_dim & 1) || rotary_dim > D ||
+      (cos_sin && (half % 64 != 0 || half <= 0)))
+    return (int)hipErrorInvalidValue;
+#define ROPE_PARTS_CASE(E, NP)                                                                             \
+  if (D == 64 * E && n_parts == NP)                                                                        \
+    return launch_rope_parts<bf16_t, E, NP>(qkv, parts, part_stride, slot_mapping, q_w, k_w, eps, cos_sin, \
+                                            rotary_dim, k_pages, v_pages, page_size, n_tokens, nq, nkv, stream);
+  ROPE_PARTS_CASE(2, 2) ROPE_PARTS_CASE(2, 3) ROPE_PARTS_CASE(2, 4)
+  ROPE_PARTS_CASE(4, 2) ROPE_PARTS_CASE(4, 3) ROPE_PARTS_CASE(4, 4)
+#undef ROPE_PARTS_CASE
+  return (int)hipErrorInvalidValue;
+}

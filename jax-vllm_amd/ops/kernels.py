@@ -83,7 +83,8 @@ def add_rmsnorm(h, delta, weight, out, eps: float, rows=None) -> None:
 
     Without ``rows``: h += delta (in place, float), out = norm(h) * weight for every row.
     With ``rows`` (int32 indices): out[i] = norm(h[rows[i]] + delta[rows[i]]) * weight and
-    h is left as it is.  ``delta`` may be None.
+    h is left as it is.  ``delta`` may be None, or a float32 stack [parts, rows of h, hidden] of
+    partial products (``linear(..., partial_ok=True)``), which are added in their order.
     """
     _dev(h, delta, weight, out, rows)
     _f32(h, "h")
@@ -91,12 +92,23 @@ def add_rmsnorm(h, delta, weight, out, eps: float, rows=None) -> None:
     _f32(weight, "weight", hidden)
     n_out = out.shape[0]
     _need(out.shape[-1] == hidden, "out width differs from h")
-    if delta is not None:
-        _need(delta.shape == h.shape and delta.dtype == out.dtype, "delta must match h's shape and out's type")
     if rows is None:
         _need(n_out == h.shape[0], "out must have one row per row of h")
     else:
         _i32(rows, "rows", n_out)
+    if delta is not None and delta.dim() == 3:
+        _need(delta.dtype == torch.float32 and delta.shape[1:] == h.shape and delta.shape[0] <= 4,
+              "partial products must be float32 [parts <= 4, *h.shape]")
+        _need(hidden % 4 == 0 and hidden <= PARTIAL_SUM_MAX_WIDTH, "partial products need a width that is a multiple of 4, at most 8192")
+        fn = getattr(library.core(), f"jv_add_rmsnorm_parts_{_suffix(out.dtype)}")
+        _check(
+            fn(_ptr(h), _ptr(delta), c_int(delta.shape[0]), c_longlong(delta.stride(0)), _ptr(weight), _ptr(out),
+               _ptr(rows), c_int(n_out), c_int(hidden), c_float(eps), _stream()),
+            "add_rmsnorm",
+        )
+        return
+    if delta is not None:
+        _need(delta.shape == h.shape and delta.dtype == out.dtype, "delta must match h's shape and out's type")
     fn = getattr(library.core(), f"jv_add_rmsnorm_{_suffix(out.dtype)}")
     _check(
         fn(_ptr(h), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows), c_int(n_out), c_int(hidden),
@@ -173,12 +185,20 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, out=None) -> tor
     return out
 
 
+def rope_takes_parts(dtype, head_dim: int, interleaved: bool, rotary_dim: int, rotated: bool) -> bool:
+    """Whether ``qk_norm_rope_write`` takes its input as float partial products (``parts``)."""
+    return (dtype == torch.bfloat16 and head_dim in (128, 256) and not interleaved
+            and (not rotated or (rotary_dim % 128 == 0 and rotary_dim > 0)))
+
+
 def qk_norm_rope_write(qkv, slot_mapping, q_weight, k_weight, eps, cos_sin, rotary_dim, interleaved,
-                       k_pages, v_pages, page_size, nq, nkv, head_dim) -> None:
+                       k_pages, v_pages, page_size, nq, nkv, head_dim, parts=None) -> None:
     """Per-head q/k RMSNorm (if weights given), rotation (if a ``rope_table`` is given), q in
     place, k and v into their pages (if pages given): K [pages, nkv, page_size, D], V transposed
-    [pages, nkv, D, page_size]."""
-    _dev(qkv, slot_mapping, q_weight, k_weight, cos_sin, k_pages, v_pages)
+    [pages, nkv, D, page_size].  With ``parts`` (float32 [2..4, tokens, (nq + 2 nkv) * D], see
+    ``linear(..., partial_ok=True)``) the input is the sum of the parts, added in order, and
+    ``qkv`` only receives the q heads."""
+    _dev(qkv, slot_mapping, q_weight, k_weight, cos_sin, k_pages, v_pages, parts)
     n = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.shape[1] == (nq + 2 * nkv) * head_dim, "qkv must be [tokens, (nq + 2 nkv) * D]")
     _need(head_dim <= 512, "head size above 512 is not supported by the rotation kernel")
@@ -192,6 +212,20 @@ def qk_norm_rope_write(qkv, slot_mapping, q_weight, k_weight, eps, cos_sin, rota
     if k_pages is not None:
         _i32(slot_mapping, "slot_mapping", n)
         _check_pages(k_pages, v_pages, qkv.dtype, nkv, page_size, head_dim)
+    if parts is not None:
+        _need(rope_takes_parts(qkv.dtype, head_dim, interleaved, rotary_dim, cos_sin is not None),
+              "partial products are taken for bfloat16, head size 128 or 256, half-split pairing, full rotation")
+        _need(parts.dtype == torch.float32 and parts.dim() == 3 and 2 <= parts.shape[0] <= 4
+              and parts.shape[1:] == qkv.shape, "parts must be float32 [2..4, tokens, (nq + 2 nkv) * D]")
+        _check(
+            library.core().jv_qk_norm_rope_write_parts_bf16(
+                _ptr(qkv), _ptr(parts), c_int(parts.shape[0]), c_longlong(parts.stride(0)),
+                _ptr(slot_mapping if k_pages is not None else None), _ptr(q_weight), _ptr(k_weight), c_float(eps),
+                _ptr(cos_sin), c_int(rotary_dim if cos_sin is not None else 0), _ptr(k_pages), _ptr(v_pages),
+                c_int(page_size), c_int(n), c_int(nq), c_int(nkv), c_int(head_dim), _stream()),
+            "qk_norm_rope_write",
+        )
+        return
     fn = getattr(library.core(), f"jv_qk_norm_rope_write_{_suffix(qkv.dtype)}")
     _check(
         fn(_ptr(qkv), _ptr(slot_mapping if k_pages is not None else None), _ptr(q_weight), _ptr(k_weight),
@@ -250,15 +284,20 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out=None) -> torch.Tensor:
 
 SKINNY_MAX_ROWS = 64
 SKINNY_AUTO_ROWS = 16   # up to here ``linear`` prefers the streaming kernel to the library
+PARTIAL_SUM_MAX_WIDTH = 8192        # widest row whose partial products the norm kernel adds
+PARTIAL_BLOCKS = 1024               # a streaming product wants about this many blocks
+PARTIAL_SHAPE = (-1, 4, 4)          # block shape of products whose inner size is shared out: phases of 512 columns
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_pairs: bool = False,
-                block_shape=(0, 0, 0), out=None) -> torch.Tensor:
+                block_shape=(0, 0, 0), out=None, ksplit: int = 1) -> torch.Tensor:
     """x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w [N, K]: the weight-streaming
     product of decode steps.  With ``silu_pairs`` the rows of w alternate gate and up rows and
     the result is silu(x.w[2j]) * (x.w[2j+1]), bfloat16 [M, N/2].  Output bfloat16 or float32.
     ``block_shape``: (row tiles, K slices, MFMA steps per iteration) of a block, zeros: chosen
-    from the shape; (-1, waves, pieces) selects the organisation with x resident in LDS."""
+    from the shape; (-1, waves, pieces) selects the organisation with x resident in LDS.
+    ``ksplit`` > 1 (that organisation, float32 output): the inner size is shared out to so many
+    blocks per row tile and the result is [ksplit, M, N], partial products to be added in order."""
     _dev(x, w, out)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     m = x.shape[0]
@@ -269,15 +308,19 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
     _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
           "the silu epilogue writes bfloat16, needs an even number of rows of w and the chunked organisation")
+    _need(ksplit >= 1 and (ksplit == 1 or (block_shape[0] == -1 and out_dtype == torch.float32 and m <= 16)),
+          "sharing the inner size out needs the resident organisation, float32 output and at most 16 rows")
     n_out = n // 2 if silu_pairs else n
+    shape = (m, n_out) if ksplit == 1 else (ksplit, m, n_out)
     if out is None:
-        out = torch.empty((m, n_out), dtype=out_dtype, device=x.device)
-    _need(out.shape == (m, n_out) and out.dtype == out_dtype, "out must be [M, N] (or [M, N/2]) of the output type")
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    _need(out.shape == shape and out.dtype == out_dtype and out.is_contiguous(),
+          "out must be [M, N] (or [M, N/2], or [ksplit, M, N]) of the output type")
     _check(
         library.core().jv_gemm_skinny_bf16(
-            _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.shape[1]), c_longlong(n_out),
+            _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.stride(0)), c_longlong(n_out),
             c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_pairs else 0),
-            c_int(block_shape[0]), c_int(block_shape[1]), c_int(block_shape[2]), _stream()),
+            c_int(block_shape[0]), c_int(block_shape[1]), c_int(block_shape[2]), c_int(ksplit), _stream()),
         "gemm_skinny",
     )
     return out
@@ -289,18 +332,38 @@ def skinny_applies(x: torch.Tensor, w: torch.Tensor) -> bool:
         and w.shape[1] % 8 == 0
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None) -> torch.Tensor:
+def partial_split(m: int, n: int, k: int) -> int:
+    """Into how many parts ``linear(..., partial_ok=True)`` shares out the inner size: a matrix with
+    few rows gives too few blocks to keep the memory system busy (measured: 33 MB stream in 12 us
+    from 256 blocks, in 7 us from 1,024), so its columns are shared out to up to 4 blocks per row tile."""
+    tiles = -(-n // 16)
+    phases = -(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32))
+    if m > SKINNY_AUTO_ROWS or n % 4 or n > PARTIAL_SUM_MAX_WIDTH or tiles * 2 > PARTIAL_BLOCKS:
+        return 1
+    parts = min(4, -(-PARTIAL_BLOCKS // tiles))
+    if parts == 3:
+        parts = 4
+    return max(1, min(parts, phases))
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = False) -> torch.Tensor:
     """x @ w.T for w stored [out, in].
 
     float32: the library's own float-FMA kernel (no reduced-precision matrix mode).
-    bfloat16, at most 64 rows: the weight-streaming MFMA kernel of this library.
+    bfloat16, at most 16 rows: the weight-streaming MFMA kernel of this library.
     bfloat16, more rows: a plain library matrix product (hipBLASLt through torch), float accumulation.
+    With ``partial_ok`` the caller takes a float32 stack [parts, M, N] of partial products as well
+    (to be added in order, as ``add_rmsnorm`` does); it is returned for narrow matrices at few rows.
     """
     if x.dtype == torch.float32:
         y = gemm_f32(x, w)
     else:
         _need(x.dtype == w.dtype, "x and w must have one type")
         if skinny_applies(x, w):
+            if partial_ok and out_dtype in (None, torch.bfloat16):
+                parts = partial_split(x.shape[0], w.shape[0], w.shape[1])
+                if parts > 1:
+                    return gemm_skinny(x, w, torch.float32, block_shape=PARTIAL_SHAPE, ksplit=parts)
             return gemm_skinny(x, w, out_dtype or torch.bfloat16)
         y = torch.mm(x, w.t())
     if out_dtype is not None and y.dtype != out_dtype:

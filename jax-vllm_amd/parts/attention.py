@@ -64,22 +64,27 @@ class GroupedQueryAttention:
     # ---- one step
     def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
         n = x.shape[0]
-        qkv = K.linear(x, self.w_qkv)
         cos_sin, rotary_dim, interleaved = (
             self.position.fused_arguments(ctx) if self.position is not None else (None, 0, False)
         )
+        # at few rows the projection may come as float partial products, which the next kernel adds
+        qkv = K.linear(x, self.w_qkv, partial_ok=K.rope_takes_parts(x.dtype, self.d, interleaved, rotary_dim,
+                                                                    cos_sin is not None))
+        parts = None
+        if qkv.dim() == 3:
+            parts, qkv = qkv, torch.empty(qkv.shape[1:], dtype=x.dtype, device=x.device)
         writes = mem.writes
         K.qk_norm_rope_write(
             qkv, ctx.slot_mappings[mem.group] if writes else None, self.q_norm, self.k_norm,
             self.qk_norm_eps or 0.0, cos_sin, rotary_dim, interleaved,
             mem.k_pages if writes else None, mem.v_pages if writes else None, ctx.page_size,
-            self.nq, self.nkv, self.d,
+            self.nq, self.nkv, self.d, parts=parts,
         )
         out = torch.empty((n, self.nq * self.d), dtype=x.dtype, device=x.device)
         from . import attention_backend
 
         attention_backend.run(self, out, qkv, ctx, mem)
-        return K.linear(out, self.w_o)
+        return K.linear(out, self.w_o, partial_ok=True)   # the next norm adds the partial products
 
 
 register_part("mixer", "gqa_attention", GroupedQueryAttention)

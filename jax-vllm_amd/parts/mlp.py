@@ -36,7 +36,7 @@ class GatedMLP:
             z = K.gemm_skinny(x, self.w_gate_up, x.dtype, silu_pairs=True)
         else:
             z = K.silu_mul(K.linear(x, self.w_gate_up), interleaved=True)
-        return K.linear(z, self.w_down)
+        return K.linear(z, self.w_down, partial_ok=True)   # the next norm adds the partial products
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

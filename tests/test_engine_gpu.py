@@ -216,6 +216,17 @@ def test_parts_alone(dtype):
     out = norm.add_norm(h, delta.cuda())
     torch.testing.assert_close(h.cpu(), x + delta.float())
     torch.testing.assert_close(out.float().cpu(), P.rms_norm(wn, 1e-4, x + delta.float()), **tol)
+    # the delta as a stack of float partial products: added in order, then to the residual
+    h3 = x.clone().cuda()
+    parts = torch.randn(3, t, hidden, generator=g)
+    out3 = norm.add_norm(h3, parts.cuda())
+    total = (parts[0] + parts[1]) + parts[2]
+    torch.testing.assert_close(h3.cpu(), x + total, rtol=0, atol=0)
+    torch.testing.assert_close(out3.float().cpu(), P.rms_norm(wn, 1e-4, x + total), **tol)
+    rows = torch.tensor([4, 0], dtype=torch.int32).cuda()
+    out_rows = norm.add_norm(h3, parts.cuda(), rows=rows)   # selected rows only, h untouched
+    torch.testing.assert_close(h3.cpu(), x + total, rtol=0, atol=0)
+    torch.testing.assert_close(out_rows.float().cpu(), P.rms_norm(wn, 1e-4, (x + total + total)[[4, 0]]), **tol)
     torch.testing.assert_close(norm.forward(x.to(dtype).cuda()).float().cpu(), P.rms_norm(wn, 1e-4, x.to(dtype).float()), **tol)
 
     mlp = build_part("feed_forward", PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter}))
@@ -225,7 +236,11 @@ def test_parts_alone(dtype):
     for rows in (t, 70):   # few rows (streaming kernel) and many (library product)
         xi = torch.randn(rows, hidden, generator=g).to(dtype)
         ref = P.swiglu(ws["gate_proj.weight"].float(), ws["up_proj.weight"].float(), ws["down_proj.weight"].float(), xi.float())
-        torch.testing.assert_close(mlp.forward(xi.cuda()).float().cpu(), ref, **tol)
+        got = mlp.forward(xi.cuda())
+        if got.dim() == 3:                     # a stack of float partial products, added by the next norm
+            assert got.dtype == torch.float32
+            got = got.sum(0)
+        torch.testing.assert_close(got.float().cpu(), ref, **tol)
 
     emb = build_part("embedding", PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": hidden}))
     table = torch.randn(vocab, hidden, generator=g).to(dtype)
@@ -300,6 +315,8 @@ def test_attention_part_alone(folders, dtype):
         out = att.forward(torch.cat([x for _, x in parts]).cuda(), ctx, mem)
         for r, x in parts:
             cache.commit(r, [0] * x.shape[0])
+        if out.dim() == 3:                     # float partial products of the output projection
+            out = out.sum(0)
         return out.float().cpu()
 
     tol = dict(rtol=2e-5, atol=2e-5) if dtype == "float32" else dict(rtol=3e-2, atol=3e-2)

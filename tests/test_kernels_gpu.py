@@ -183,6 +183,47 @@ def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_nor
     torch.testing.assert_close(qkv2.float().view(t, nq + 2 * nkv, d)[:, :nq], got_q, rtol=0, atol=0)
 
 
+@pytest.mark.parametrize("nq,nkv,d,n_parts,t,with_norm", [(6, 2, 128, 2, 5, True), (4, 4, 256, 4, 16, True),
+                                                         (32, 8, 128, 4, 8, True), (3, 1, 128, 3, 9, False)])
+def test_qk_norm_rope_write_from_partial_products(nq, nkv, d, n_parts, t, with_norm):
+    """The projection arrives as float partial products: their ordered sum must give what the
+    whole bfloat16 projection gives, up to the rounding the whole one has and the parts do not."""
+    bf = torch.bfloat16
+    page_size, eps, width = 8, 1e-6, (nq + 2 * nkv) * d
+    pages = t + 2
+    parts = randn(n_parts, t, width, seed=40, scale=0.7)
+    whole = (parts[0].cpu() + parts[1].cpu())
+    for q in range(2, n_parts):
+        whole = whole + parts[q].cpu()
+    g = torch.Generator().manual_seed(t)
+    pos = torch.randint(0, 3000, (t,), generator=g).to(torch.int32).cuda()
+    slots = (torch.randperm((pages - 1) * page_size, generator=g)[:t] + page_size).to(torch.int32).cuda()
+    qw = (1 + 0.1 * randn(d, seed=12)) if with_norm else None
+    kw = (1 + 0.1 * randn(d, seed=13)) if with_norm else None
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).cuda()
+    table = K().rope_table(pos, inv_freq)
+    outs = []
+    for use_parts in (True, False):
+        k_pages = torch.zeros(pages, nkv, page_size, d, dtype=bf).cuda()
+        v_pages = torch.zeros(pages, nkv, d, page_size, dtype=bf).cuda()
+        qkv = torch.zeros(t, width, dtype=bf).cuda() if use_parts else whole.to(bf).cuda()
+        K().qk_norm_rope_write(qkv, slots, qw, kw, eps, table, d, False, k_pages, v_pages, page_size, nq, nkv, d,
+                               parts=parts if use_parts else None)
+        outs.append((qkv.float().view(t, nq + 2 * nkv, d)[:, :nq].cpu(), k_pages.float().cpu(), v_pages.float().cpu()))
+    for a, b in zip(*outs):
+        torch.testing.assert_close(a, b, rtol=3e-2, atol=3e-2)
+    # and against the float formula directly
+    x = whole.view(t, nq + 2 * nkv, d)
+    qf = x[:, :nq]
+    if with_norm:
+        qf = qf * torch.rsqrt((qf * qf).mean(-1, keepdim=True) + eps) * qw.cpu()
+    qf = rope_reference(qf.cuda(), pos, inv_freq, d, False).cpu()
+    torch.testing.assert_close(outs[0][0], qf, rtol=1e-2, atol=1e-2)
+    assert not K().rope_takes_parts(torch.bfloat16, 64, False, 64, True)
+    assert not K().rope_takes_parts(torch.bfloat16, 128, True, 128, True)
+    assert not K().rope_takes_parts(torch.float32, 128, False, 128, True)
+
+
 # ------------------------------------------------------------------ paged attention
 def build_paged(k, v, page_size, seed=0, extra_pages=3):
     """Scatter per-request [T, nkv, D] keys/values over shuffled pages; returns pages and tables."""
@@ -585,6 +626,29 @@ def test_gemm_skinny(m, n, k, shape, out_dtype):
         one = K().gemm_skinny(x[2:3].contiguous() if m > 2 else x[:1].contiguous(), w, out_dtype, block_shape=shape)
         exact = dict(rtol=0, atol=0) if shape != (0, 0, 0) else dict(rtol=1e-2, atol=1e-3)
         torch.testing.assert_close(one, out[2:3] if m > 2 else out[:1], **exact)
+
+
+@pytest.mark.parametrize("m,n,k,shape,ksplit", [(8, 4096, 4096, (-1, 4, 4), 4), (1, 100, 12288, (-1, 4, 4), 4),
+                                                (16, 333, 1000, (-1, 8, 2), 2), (5, 64, 2560, (-1, 4, 4), 3),
+                                                (3, 48, 1000, (-1, 2, 2), 4)])
+def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
+    """Partial products [ksplit, M, N] in float: part s covers its own columns only, and the
+    ordered sum is the product."""
+    x = randn(m, k, dtype=torch.bfloat16, seed=34, scale=0.5)
+    w = randn(n, k, dtype=torch.bfloat16, seed=35, scale=0.5)
+    parts = K().gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=ksplit)
+    assert parts.shape == (ksplit, m, n) and parts.dtype == torch.float32
+    kp = shape[1] * shape[2] * 32
+    k_per = -(-(-(-k // kp)) // ksplit) * kp
+    for s in range(ksplit):
+        lo, hi = s * k_per, min(k, (s + 1) * k_per)
+        ref = x[:, lo:hi].double() @ w[:, lo:hi].double().T
+        torch.testing.assert_close(parts[s].double().cpu(), ref.cpu(), rtol=1e-4, atol=1e-3)
+    again = K().gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=ksplit)
+    assert torch.equal(parts, again)
+    from jax_vllm_amd.ops.kernels import KernelArgumentError
+    with pytest.raises((KernelArgumentError, RuntimeError)):
+        K().gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=1000)   # more parts than phases
 
 
 @pytest.mark.parametrize("m,inter,k", [(1, 176, 80), (8, 12288, 96), (40, 224, 104), (16, 1000, 4096)])
