@@ -23,12 +23,15 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define SK_PAD 8  // bf16 elements of padding per LDS row (keeps 16-byte reads of 16 rows off the same banks)
 
+// Up to 16 waves for one tile of x rows (128 registers a lane); at most 8 beyond, where the
+// accumulators, the B operands and the x pieces in flight need more.
 template <int MT, int NKS, typename OutT, bool PAIRS>
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(MT == 1 ? 1024 : 512)
 gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
                    int M, int N, int K, long long ldx, long long ldy, int WR, int WK) {
   constexpr int STEP = NKS * 32;
   constexpr int ROWS = MT * 16;
+  constexpr int XP = 2 * MT;                 // x pieces a thread keeps in flight
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int KCB = WK * STEP;                 // columns of one x chunk
   const int LROW = KCB + SK_PAD;             // LDS row length in elements
@@ -79,29 +82,45 @@ gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
   for (int it = 0; it < n_iter; ++it) {
     const bool more = it + 1 < n_iter;
     if (more) load_w(it + 1, a_nxt);
-    // next chunk's pieces of this thread: at most 2 in flight in registers, the rest (large M
-    // with few threads) are copied after the products
-    bf16x8 xr0 = zero, xr1 = zero;
-    const int c0 = tid, c1 = tid + nthreads;
+    // next chunk's pieces of this thread: up to XP in flight in registers while this chunk is
+    // multiplied; what is beyond (many rows, few threads) is copied after the products
+    bf16x8 xr[XP];
     if (more) {
-      if (c0 < xvecs) xr0 = load_x_piece(it + 1, c0);
-      if (c1 < xvecs) xr1 = load_x_piece(it + 1, c1);
+#pragma unroll
+      for (int i = 0; i < XP; ++i) {
+        const int c = tid + i * nthreads;
+        xr[i] = c < xvecs ? load_x_piece(it + 1, c) : zero;
+      }
     }
     __syncthreads();  // buffer it&1 is complete; everyone is done reading buffer (it+1)&1
     const bf16_t* xb = xs + ((it & 1) * ROWS) * LROW + wk * STEP + lc * 8;
+    // the B operands of one 32-column step are read a step ahead of their products (the fence
+    // keeps the compiler from moving each read down to its product, which would then wait a full
+    // LDS round trip every time)
+    bf16x8 bfr[2][MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) bfr[0][mt] = *(const bf16x8*)(xb + (mt * 16 + li) * LROW);
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
+      if (ks + 1 < NKS) {
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8 b = *(const bf16x8*)(xb + (mt * 16 + li) * LROW + ks * 32);
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[ks], b, acc[mt], 0, 0, 0);
+        for (int mt = 0; mt < MT; ++mt)
+          bfr[(ks + 1) & 1][mt] = *(const bf16x8*)(xb + (mt * 16 + li) * LROW + (ks + 1) * 32);
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_cur[ks], bfr[ks & 1][mt], acc[mt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (more) {
       const int nb = (it + 1) & 1;
-      if (c0 < xvecs) store_x_piece(nb, c0, xr0);
-      if (c1 < xvecs) store_x_piece(nb, c1, xr1);
-      for (int c = tid + 2 * nthreads; c < xvecs; c += nthreads) store_x_piece(nb, c, load_x_piece(it + 1, c));
+#pragma unroll
+      for (int i = 0; i < XP; ++i) {
+        const int c = tid + i * nthreads;
+        if (c < xvecs) store_x_piece(nb, c, xr[i]);
+      }
+      for (int c = tid + XP * nthreads; c < xvecs; c += nthreads) store_x_piece(nb, c, load_x_piece(it + 1, c));
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) a_cur[ks] = a_nxt[ks];
     }
@@ -116,8 +135,12 @@ gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     for (int mt = 0; mt < MT; ++mt) *(f32x4*)(red + (((wk * WR + wr) * MT + mt) * 256 + lane * 4)) = acc[mt];
     __syncthreads();
   }
-  // the WK waves of one row tile share its MT column tiles out between them
-  for (int mt = wk; mt < MT; mt += WK) {
+  // the WK waves of one row tile share its MT column tiles out between them (the loop is
+  // unrolled over constant mt: a run-time index would put the accumulators into scratch
+  // memory for the whole kernel)
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    if (mt % WK != wk) continue;
     f32x4 s = WK > 1 ? *(const f32x4*)(red + ((wr * MT + mt) * 256 + lane * 4)) : acc[mt];
     for (int w = 1; w < WK; ++w) {
       const f32x4 t = *(const f32x4*)(red + (((w * WR + wr) * MT + mt) * 256 + lane * 4));
@@ -358,7 +381,7 @@ extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M,
   if (wk <= 0) wk = cwk;
   if (nks <= 0) nks = cnks;
   const int MT = (M + 15) / 16;
-  if (wr * wk > 16 || (nks != 2 && nks != 4 && nks != 8)) return (int)hipErrorInvalidValue;
+  if (wr * wk > (MT == 1 ? 16 : 8) || (nks != 2 && nks != 4 && nks != 8)) return (int)hipErrorInvalidValue;
   if (skinny_shmem(MT, nks, wr, wk) > 160 * 1024) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
   if (silu_pairs) return dispatch_nks<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);

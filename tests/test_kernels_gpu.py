@@ -607,7 +607,7 @@ def test_mfma_attention_refuses_what_it_cannot_do():
 @pytest.mark.parametrize("m,n,k,shape", [
     (1, 96, 64, (0, 0, 0)), (8, 224, 96, (0, 0, 0)), (33, 520, 136, (2, 3, 2)), (64, 100, 4096, (0, 0, 0)),
     (5, 777, 80, (1, 16, 2)), (17, 64, 12288, (1, 8, 4)), (3, 30, 264, (1, 1, 8)), (16, 48, 2056, (0, 0, 0)),
-    (8, 24576, 512, (0, 0, 0)), (48, 6144, 1024, (4, 4, 2)), (1, 6144, 4096, (1, 8, 4)), (9, 160, 4096, (4, 4, 8)),
+    (8, 24576, 512, (0, 0, 0)), (48, 6144, 1024, (4, 2, 2)), (1, 6144, 4096, (1, 8, 4)), (9, 160, 4096, (4, 4, 8)),
     (1, 8200, 4096, (0, 0, 0)), (2, 100, 4096, (-1, 8, 16)), (8, 333, 1000, (-1, 16, 4)), (16, 64, 12288, (-1, 4, 8)),
     (11, 50, 72, (-1, 3, 4))])
 def test_gemm_skinny(m, n, k, shape, out_dtype):
