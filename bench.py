@@ -47,11 +47,11 @@ def sync():
     torch.cuda.synchronize()
 
 
-def measure_decode(llm, batch, steps, warmup, rng, vocab):
+def measure_decode(llm, batch, steps, warmup, rng, vocab, prompt_len=PROMPT_LEN):
     """Tokens/s of ``steps`` decode steps at ``batch`` after prefilling 1,024-token prompts."""
     from jax_vllm_amd import SamplingParams
 
-    prompts = [rng.integers(0, vocab, size=PROMPT_LEN).tolist() for _ in range(batch)]
+    prompts = [rng.integers(0, vocab, size=prompt_len).tolist() for _ in range(batch)]
     sp = SamplingParams(max_new_tokens=warmup + steps + 128)
     for p in prompts:
         llm.add_request(p, sp)
@@ -104,6 +104,8 @@ def main():
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
                     help="run one phase alone and print its result (for profiling)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
+                    help="with --only decode: prompt length of the decoding requests (long-context runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -122,7 +124,8 @@ def main():
     max_batch = args.batch if (args.skip_points or args.only) else max(64, args.batch)
     block = 16
     llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=max_batch,
-              max_model_len=MAX_CONTEXT, num_blocks=1 + max_batch * (-(-(PROMPT_LEN + 2 * 1024) // block)),
+              max_model_len=max(MAX_CONTEXT, args.prompt_len + 2 * 1024),
+              num_blocks=1 + max_batch * (-(-(args.prompt_len + 2 * 1024) // block)),
               max_num_batched_tokens=max(PREFILL_TOKENS, max_batch), enable_prefix_cache=False)
     itemsize = 2 if args.dtype == "bf16" else 4
     wbytes, per_layer_params = weight_bytes(cfg, layers, itemsize)
@@ -133,7 +136,7 @@ def main():
         print(json.dumps({"prefill_ms": round(pre_s * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}), flush=True)
         return
     if args.only == "decode":
-        tps, step_s, mean_ctx = measure_decode(llm, args.batch, args.steps, args.warmup, rng, vocab)
+        tps, step_s, mean_ctx = measure_decode(llm, args.batch, args.steps, args.warmup, rng, vocab, args.prompt_len)
         print(json.dumps({"decode_tokens_per_s": round(tps, 1), "ms_per_step": round(step_s * 1e3, 4),
                           "batch": args.batch, "mean_context": round(mean_ctx, 1), "layers": layers}), flush=True)
         return

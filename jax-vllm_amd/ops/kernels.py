@@ -481,17 +481,3 @@ def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_se
                            _stream()),
         "attn_decode_mfma",
     )
-
-
-# --------------------------------------------------------------------------- cache warming
-_prefetch_sink = {}
-
-
-def prefetch(t: torch.Tensor, blocks: int = 64) -> None:
-    """Reads a tensor's bytes with a few workgroups so that they sit in the memory-side cache."""
-    _dev(t)
-    sink = _prefetch_sink.get(t.device)
-    if sink is None:
-        sink = _prefetch_sink[t.device] = torch.zeros(1, dtype=torch.float32, device=t.device)
-    _check(library.core().jv_prefetch(_ptr(t), c_longlong(t.numel() * t.element_size()), c_int(blocks), _ptr(sink),
-                                      _stream()), "prefetch")
