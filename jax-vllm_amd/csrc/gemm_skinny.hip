@@ -330,6 +330,110 @@ static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, i
   return (int)hipErrorInvalidValue;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Third organisation, for at most 16 rows of x and an inner size of at most 8 * NL * 32: blocks
+// that stay.  Each of a block's 8 waves keeps ITS slice of x (NL steps of 32 columns) in registers
+// as MFMA B operands for the whole kernel, so the loop over the block's row tiles of W touches
+// LDS only to add the 8 waves' partial tiles: no staging of x, no barrier between the loads.
+// The next tile's weights are asked for before the current tile is multiplied and reduced.
+// A longer inner size is shared out to gridDim.y groups of blocks, 8 * NL * 32 columns each,
+// which write float partial products to y + group * M * ldy (added by the reader, in order).
+template <int NL, typename OutT, bool PAIRS>
+__global__ void __launch_bounds__(512)
+gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
+                              int M, int N, int K, long long ldx, long long ldy) {
+  y += (long long)blockIdx.y * M * ldy;
+  __shared__ __attribute__((aligned(16))) float red[8 * 256];
+  const int tid = threadIdx.x;
+  const int wk = tid >> 6, lane = tid & 63, li = lane & 15, lc = lane >> 4;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int k0 = (blockIdx.y * 8 + wk) * NL * 32 + lc * 8;     // this lane's first column
+  const int n_tiles = (N + 15) / 16;
+  // x: row li (zero beyond M), this wave's columns
+  bf16x8 b[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int k = k0 + i * 32;
+    b[i] = (li < M && k < K) ? *(const bf16x8*)(x + (long long)li * ldx + k) : zero;
+  }
+  auto load_tile = [&](int tile, bf16x8 (&a)[NL]) {
+    const int n = tile * 16 + li;
+    const bf16_t* wrow = W + (long long)(n < N ? n : 0) * K + k0;
+#pragma unroll
+    for (int i = 0; i < NL; ++i) a[i] = (n < N && k0 + i * 32 < K) ? *(const bf16x8*)(wrow + i * 32) : zero;
+  };
+  auto finish_tile = [&](int tile, bf16x8 (&a)[NL]) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NL; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[i], acc, 0, 0, 0);
+    *(f32x4*)(red + (wk * 256 + lane * 4)) = acc;
+    __syncthreads();
+    if (wk == 0) {
+      f32x4 s = acc;                               // fixed order: wave 0, 1, ..., 7
+#pragma unroll
+      for (int w = 1; w < 8; ++w) {
+        const f32x4 t = *(const f32x4*)(red + (w * 256 + lane * 4));
+        s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
+      }
+      const int nb = tile * 16 + lc * 4;           // the accumulator holds y^T[n = lc*4+e][m = li]
+      if (li < M) {
+        if (PAIRS) {
+#pragma unroll
+          for (int e = 0; e < 4; e += 2)
+            if (nb + e + 1 < N)
+              y[(long long)li * ldy + (nb + e) / 2] = from_f32<OutT>(s[e] / (1.f + expf(-s[e])) * s[e + 1]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (nb + e < N) y[(long long)li * ldy + nb + e] = from_f32<OutT>(s[e]);
+        }
+      }
+    }
+    __syncthreads();                               // red may be written again
+  };
+  bf16x8 a0[NL], a1[NL];
+  int tile = blockIdx.x;
+  if (tile < n_tiles) load_tile(tile, a0);
+  while (tile < n_tiles) {
+    int next = tile + gridDim.x;
+    if (next < n_tiles) load_tile(next, a1);
+    finish_tile(tile, a0);
+    tile = next;
+    if (tile >= n_tiles) break;
+    next = tile + gridDim.x;
+    if (next < n_tiles) load_tile(next, a0);
+    finish_tile(tile, a1);
+    tile = next;
+  }
+}
+
+template <int NL, typename OutT, bool PAIRS>
+static int launch_persistent(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
+                             long long ldy, int blocks, int ksplit, hipStream_t stream) {
+  const int n_tiles = (N + 15) / 16;
+  blocks = (blocks + ksplit - 1) / ksplit;           // per group
+  if (blocks > n_tiles) blocks = n_tiles;
+  hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, OutT, PAIRS>), dim3(blocks, ksplit), dim3(512), 0, stream,
+                     (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
+  return JV_LAUNCH_CHECK();
+}
+
+// wr == -2: nks = NL in {4, 8, 16}, wk = blocks in all; the inner size must be at most
+// ksplit * 8 * NL * 32 and more than (ksplit - 1) * 8 * NL * 32
+template <typename OutT, bool PAIRS>
+static int dispatch_persistent(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
+                               long long ldy, int blocks, int ksplit, hipStream_t s) {
+  if (M > 16 || blocks < 1 || ksplit > 65535 || K > (long long)ksplit * 8 * nl * 32 ||
+      K <= (long long)(ksplit - 1) * 8 * nl * 32)
+    return (int)hipErrorInvalidValue;
+  switch (nl) {
+    case 4: return launch_persistent<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 8: return launch_persistent<8, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 16: return launch_persistent<16, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+  }
+  return (int)hipErrorInvalidValue;
+}
+
 // Shape of the block chosen from the problem.  Measured on MI355X (weights beyond the last-level
 // cache): one row tile per block with 8 K slices of 128 columns streams fastest for up to 16
 // rows of x at every matrix shape of an 8B-class model; more row tiles per block lose more to
@@ -354,7 +458,7 @@ static void skinny_config(int M, int N, int K, int* wr, int* wk, int* nks) {
 // wr, wk, nks: block shape (row tiles, K slices, MFMA steps per iteration); 0 picks them.
 // wr == -1 selects the resident-x organisation (M <= 16, no silu): wk waves, nks in {2, 4, 8, 16}
 // weight pieces per wave and phase.
-// ksplit > 1 (resident-x organisation, float output only): K is shared out to ksplit blocks per
+// ksplit > 1 (resident-x organisation or blocks that stay, float output only): K is shared out to ksplit blocks per
 // row tile and y is [ksplit][M][ldy], partial products that the reader adds in that order.
 extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
                                    long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
@@ -362,7 +466,13 @@ extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M,
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
   if (silu_pairs && (out_f32 || N % 2 != 0 || wr == -1)) return (int)hipErrorInvalidValue;
-  if (ksplit < 1 || (ksplit > 1 && (wr != -1 || !out_f32))) return (int)hipErrorInvalidValue;
+  if (ksplit < 1 || (ksplit > 1 && ((wr != -1 && wr != -2) || !out_f32))) return (int)hipErrorInvalidValue;
+  if (wr == -2) {   // blocks that stay: wk = number of blocks, nks = weight pieces per wave
+    hipStream_t s = (hipStream_t)stream;
+    if (silu_pairs) return dispatch_persistent<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s);
+    return out_f32 ? dispatch_persistent<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s)
+                   : dispatch_persistent<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s);
+  }
   if (wr == -1) {
     if (M > 16 || wk < 1 || wk > 16) return (int)hipErrorInvalidValue;
     hipStream_t s = (hipStream_t)stream;

@@ -284,10 +284,10 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out=None) -> torch.Tensor:
 
 SKINNY_MAX_ROWS = 64
 SKINNY_AUTO_ROWS = 16   # up to here ``linear`` prefers the streaming kernel to the library
-SKINNY_LARGE_MATRIX = 40_000_000    # elements; see skinny_applies
+SKINNY_LARGE_MATRIX = 40_000_000    # elements; see streaming_plan
 PARTIAL_SUM_MAX_WIDTH = 8192        # widest row whose partial products the norm kernel adds
 PARTIAL_BLOCKS = 1024               # a streaming product wants about this many blocks
-PARTIAL_SHAPE = (-1, 4, 4)          # block shape of products whose inner size is shared out: phases of 512 columns
+PARTIAL_SHAPE = (-1, 4, 4)          # x resident in LDS, phases of 512 columns: for inner sizes the staying blocks do not cover
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_pairs: bool = False,
@@ -296,7 +296,9 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     product of decode steps.  With ``silu_pairs`` the rows of w alternate gate and up rows and
     the result is silu(x.w[2j]) * (x.w[2j+1]), bfloat16 [M, N/2].  Output bfloat16 or float32.
     ``block_shape``: (row tiles, K slices, MFMA steps per iteration) of a block, zeros: chosen
-    from the shape; (-1, waves, pieces) selects the organisation with x resident in LDS.
+    from the shape; (-1, waves, pieces) selects the organisation with x resident in LDS;
+    (-2, blocks, pieces) the one with blocks that stay and keep x in registers (at most 16 rows,
+    inner size at most 256 * pieces).
     ``ksplit`` > 1 (that organisation, float32 output): the inner size is shared out to so many
     blocks per row tile and the result is [ksplit, M, N], partial products to be added in order."""
     _dev(x, w, out)
@@ -307,9 +309,12 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     _need(m <= SKINNY_MAX_ROWS, f"gemm_skinny takes at most {SKINNY_MAX_ROWS} rows")
     _need(k % 8 == 0, "the inner size must be a multiple of 8")
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
+    _need(block_shape[0] != -2 or (m <= 16 and block_shape[2] in (4, 8, 16)
+                                   and 256 * block_shape[2] * (ksplit - 1) < k <= 256 * block_shape[2] * ksplit),
+          "the organisation with blocks that stay takes at most 16 rows and an inner size of ksplit * 256 * pieces at most")
     _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
           "the silu epilogue writes bfloat16, needs an even number of rows of w and the chunked organisation")
-    _need(ksplit >= 1 and (ksplit == 1 or (block_shape[0] == -1 and out_dtype == torch.float32 and m <= 16)),
+    _need(ksplit >= 1 and (ksplit == 1 or (block_shape[0] in (-1, -2) and out_dtype == torch.float32 and m <= 16)),
           "sharing the inner size out needs the resident organisation, float32 output and at most 16 rows")
     n_out = n // 2 if silu_pairs else n
     shape = (m, n_out) if ksplit == 1 else (ksplit, m, n_out)
@@ -327,52 +332,88 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     return out
 
 
-def skinny_applies(x: torch.Tensor, w: torch.Tensor) -> bool:
-    """Whether ``linear`` would run the streaming kernel for these operands."""
-    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] % 8:
-        return False
-    m = x.shape[0]
-    # measured at the matrix shapes of an 8B-class model: up to 8 rows the streaming kernel wins
-    # everywhere; at 9..16 rows it still wins on small matrices (4096 x 4096: 11 against 15 us),
-    # the library on large ones (24576 x 4096: 44 against 53 us), where staging 16 rows of x per
-    # 16 rows of w costs more than the library's wider tiles
-    return m <= 8 or (m <= SKINNY_AUTO_ROWS and w.shape[0] * w.shape[1] < SKINNY_LARGE_MATRIX)
+_cu_count = {}
 
 
-def partial_split(m: int, n: int, k: int) -> int:
-    """Into how many parts ``linear(..., partial_ok=True)`` shares out the inner size: a matrix with
-    few rows gives too few blocks to keep the memory system busy (measured: 33 MB stream in 12 us
-    from 256 blocks, in 7 us from 1,024), so its columns are shared out to up to 4 blocks per row tile."""
+def _compute_units(device) -> int:
+    n = _cu_count.get(device)
+    if n is None:
+        n = _cu_count[device] = torch.cuda.get_device_properties(device).multi_processor_count
+    return n
+
+
+def _stay_pieces(k: int, parts: int):
+    """Weight pieces per wave (4, 8 or 16) with which ``parts`` groups of staying blocks cover an
+    inner size of k exactly (each group 8 waves x pieces x 32 columns), or None."""
+    for nl in (4, 8, 16):
+        if 256 * nl * (parts - 1) < k <= 256 * nl * parts:
+            return nl
+    return None
+
+
+def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok: bool = False, device=None):
+    """How ``linear`` runs a bfloat16 product at few rows: (block_shape, ksplit) for ``gemm_skinny``,
+    or None for the library.  All thresholds are measured on MI355X at the matrix shapes of an
+    8B-class model (pure reads of the same bytes: 33 MB 6.5 us, 50 MB 9.1, 101 MB 16.5, 201 MB 33.5).
+
+    * wide matrices (>= 1,024 row tiles), inner size <= 4,096, 3..16 rows: blocks that stay, one per
+      compute unit (two for very wide ones), x in registers: 201 MB in 38 us at 8 rows and 40.5 at
+      16, against 42 and 53 with x staged per block, 44 by the library;
+    * narrow matrices whose reader adds partial products: the inner size shared out to 4 groups so
+      that ~1,000 blocks stream (33 MB: 8.6 us against 11.0 from 256 blocks);
+    * one or two rows against wide matrices: x resident in LDS (chosen inside the kernel library);
+    * 9..16 rows of a large matrix that fits none of these: the library (its wider tiles amortise x);
+    * otherwise x staged chunk by chunk in LDS.
+    """
+    if m > SKINNY_AUTO_ROWS or k % 8:
+        return None
     tiles = -(-n // 16)
-    phases = -(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32))
-    if m > SKINNY_AUTO_ROWS or n % 4 or n > PARTIAL_SUM_MAX_WIDTH or tiles * 2 > PARTIAL_BLOCKS:
-        return 1
-    parts = min(4, -(-PARTIAL_BLOCKS // tiles))
-    if parts == 3:
-        parts = 4
-    return max(1, min(parts, phases))
+    cus = _compute_units(device) if device is not None else 256
+    if partial_ok and not silu_pairs and n % 4 == 0 and n <= PARTIAL_SUM_MAX_WIDTH and tiles * 2 <= PARTIAL_BLOCKS:
+        parts = min(4, -(-PARTIAL_BLOCKS // tiles))
+        parts = 4 if parts == 3 else parts
+        if parts > 1:
+            nl = _stay_pieces(k, parts)
+            if nl is not None:
+                return (-2, 2 * cus, nl), parts
+            phases = -(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32))
+            if phases >= parts and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX):
+                return PARTIAL_SHAPE, parts
+    if m >= 3 and tiles >= 4 * cus:
+        nl = _stay_pieces(k, 1)
+        if nl is not None:
+            return (-2, (2 if tiles >= 16 * cus else 1) * cus, nl), 1
+    if m > 8 and n * k >= SKINNY_LARGE_MATRIX:
+        return None
+    return (0, 0, 0), 1
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = False) -> torch.Tensor:
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = False, silu_pairs: bool = False):
     """x @ w.T for w stored [out, in].
 
     float32: the library's own float-FMA kernel (no reduced-precision matrix mode).
-    bfloat16, at most 16 rows: the weight-streaming MFMA kernel of this library.
+    bfloat16, at most 16 rows: a weight-streaming MFMA kernel of this library (``streaming_plan``).
     bfloat16, more rows: a plain library matrix product (hipBLASLt through torch), float accumulation.
     With ``partial_ok`` the caller takes a float32 stack [parts, M, N] of partial products as well
     (to be added in order, as ``add_rmsnorm`` does); it is returned for narrow matrices at few rows.
+    With ``silu_pairs`` the rows of w alternate gate and up rows and the result is
+    silu(x.w[2j]) * (x.w[2j+1]) of width N/2 (an epilogue of the streaming kernels, a kernel of
+    its own after the library's product).
     """
     if x.dtype == torch.float32:
         y = gemm_f32(x, w)
     else:
         _need(x.dtype == w.dtype, "x and w must have one type")
-        if skinny_applies(x, w):
-            if partial_ok and out_dtype in (None, torch.bfloat16):
-                parts = partial_split(x.shape[0], w.shape[0], w.shape[1])
-                if parts > 1:
-                    return gemm_skinny(x, w, torch.float32, block_shape=PARTIAL_SHAPE, ksplit=parts)
-            return gemm_skinny(x, w, out_dtype or torch.bfloat16)
+        plan = streaming_plan(x.shape[0], w.shape[0], w.shape[1], silu_pairs,
+                              partial_ok and out_dtype in (None, torch.bfloat16), x.device)
+        if plan is not None:
+            shape, parts = plan
+            if parts > 1:
+                return gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=parts)
+            return gemm_skinny(x, w, out_dtype or torch.bfloat16, silu_pairs=silu_pairs, block_shape=shape)
         y = torch.mm(x, w.t())
+    if silu_pairs:
+        return silu_mul(y, interleaved=True)
     if out_dtype is not None and y.dtype != out_dtype:
         y = y.to(out_dtype)
     return y

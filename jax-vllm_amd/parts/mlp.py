@@ -32,10 +32,7 @@ class GatedMLP:
         self.w_down = tensors["down_proj.weight"]
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
-        if K.skinny_applies(x, self.w_gate_up):
-            z = K.gemm_skinny(x, self.w_gate_up, x.dtype, silu_pairs=True)
-        else:
-            z = K.silu_mul(K.linear(x, self.w_gate_up), interleaved=True)
+        z = K.linear(x, self.w_gate_up, silu_pairs=True)    # gate and up rows alternate in the fused weight
         return K.linear(z, self.w_down, partial_ok=True)   # the next norm adds the partial products
 
 

@@ -609,7 +609,8 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     (5, 777, 80, (1, 16, 2)), (17, 64, 12288, (1, 8, 4)), (3, 30, 264, (1, 1, 8)), (16, 48, 2056, (0, 0, 0)),
     (8, 24576, 512, (0, 0, 0)), (48, 6144, 1024, (4, 2, 2)), (1, 6144, 4096, (1, 8, 4)), (9, 160, 4096, (4, 4, 8)),
     (1, 8200, 4096, (0, 0, 0)), (2, 100, 4096, (-1, 8, 16)), (8, 333, 1000, (-1, 16, 4)), (16, 64, 12288, (-1, 4, 8)),
-    (11, 50, 72, (-1, 3, 4))])
+    (11, 50, 72, (-1, 3, 4)), (8, 24576, 512, (-2, 64, 4)), (16, 333, 4096, (-2, 7, 16)), (5, 777, 2000, (-2, 1000, 8)),
+    (3, 100, 72, (-2, 3, 4)), (1, 8200, 4096, (-2, 256, 16))])
 def test_gemm_skinny(m, n, k, shape, out_dtype):
     x = randn(m, k, dtype=torch.bfloat16, seed=30, scale=0.5)
     w = randn(n, k, dtype=torch.bfloat16, seed=31, scale=0.5)
@@ -630,7 +631,8 @@ def test_gemm_skinny(m, n, k, shape, out_dtype):
 
 @pytest.mark.parametrize("m,n,k,shape,ksplit", [(8, 4096, 4096, (-1, 4, 4), 4), (1, 100, 12288, (-1, 4, 4), 4),
                                                 (16, 333, 1000, (-1, 8, 2), 2), (5, 64, 2560, (-1, 4, 4), 3),
-                                                (3, 48, 1000, (-1, 2, 2), 4)])
+                                                (3, 48, 1000, (-1, 2, 2), 4), (8, 4096, 4096, (-2, 512, 4), 4),
+                                                (16, 130, 3000, (-2, 10, 4), 3), (2, 64, 12288, (-2, 30, 16), 3)])
 def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
     """Partial products [ksplit, M, N] in float: part s covers its own columns only, and the
     ordered sum is the product."""
@@ -638,8 +640,11 @@ def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
     w = randn(n, k, dtype=torch.bfloat16, seed=35, scale=0.5)
     parts = K().gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=ksplit)
     assert parts.shape == (ksplit, m, n) and parts.dtype == torch.float32
-    kp = shape[1] * shape[2] * 32
-    k_per = -(-(-(-k // kp)) // ksplit) * kp
+    if shape[0] == -2:
+        k_per = 256 * shape[2]                   # 8 waves x pieces x 32 columns per group
+    else:
+        kp = shape[1] * shape[2] * 32
+        k_per = -(-(-(-k // kp)) // ksplit) * kp
     for s in range(ksplit):
         lo, hi = s * k_per, min(k, (s + 1) * k_per)
         ref = x[:, lo:hi].double() @ w[:, lo:hi].double().T
@@ -651,14 +656,42 @@ def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
         K().gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=1000)   # more parts than phases
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 176, 80), (8, 12288, 96), (40, 224, 104), (16, 1000, 4096)])
-def test_gemm_skinny_silu_epilogue(m, inter, k):
+def test_linear_follows_its_plan_and_all_roads_agree():
+    """``linear`` at few rows: the staying blocks, the shared-out inner size, the staged chunks and
+    the library must give the same numbers up to rounding, with and without the silu epilogue."""
+    kern = K()
+    x = randn(8, 4096, dtype=torch.bfloat16, seed=36, scale=0.5)
+    wide = randn(16640, 4096, dtype=torch.bfloat16, seed=37, scale=0.1)      # 1,040 row tiles: blocks that stay
+    narrow = randn(512, 4096, dtype=torch.bfloat16, seed=38, scale=0.1)      # 32 row tiles: inner size shared out
+    assert kern.streaming_plan(8, 16640, 4096, silu_pairs=True, device=x.device)[0][0] == -2
+    plan = kern.streaming_plan(8, 512, 4096, partial_ok=True, device=x.device)
+    assert plan[1] == 4 and kern.streaming_plan(8, 512, 4096, partial_ok=False, device=x.device) == ((0, 0, 0), 1)
+    assert kern.streaming_plan(17, 512, 4096, device=x.device) is None       # the library's
+    ref = x.double() @ narrow.double().T
+    parts = kern.linear(x, narrow, partial_ok=True)
+    assert plan[0][0] == -2 and parts.shape == (4, 8, 512) and parts.dtype == torch.float32
+    torch.testing.assert_close(parts.sum(0).double(), ref, rtol=1e-3, atol=1e-2)
+    torch.testing.assert_close(kern.linear(x, narrow).double(), ref, rtol=2e-2, atol=5e-2)
+    g, u = wide[0::2].double(), wide[1::2].double()
+    ref_act = torch.nn.functional.silu(x.double() @ g.T) * (x.double() @ u.T)
+    for rows in (8, 40):                                                    # staying blocks; library + silu kernel
+        xi = x if rows == 8 else randn(rows, 4096, dtype=torch.bfloat16, seed=39, scale=0.5)
+        want = ref_act if rows == 8 else torch.nn.functional.silu(xi.double() @ g.T) * (xi.double() @ u.T)
+        got = kern.linear(xi, wide, silu_pairs=True)
+        assert got.shape == (rows, 8320) and got.dtype == torch.bfloat16
+        torch.testing.assert_close(got.double(), want, rtol=2e-2, atol=5e-2)
+
+
+@pytest.mark.parametrize("m,inter,k,shape", [(1, 176, 80, (0, 0, 0)), (8, 12288, 96, (0, 0, 0)), (40, 224, 104, (0, 0, 0)),
+                                             (16, 1000, 4096, (0, 0, 0)), (8, 1000, 4096, (-2, 256, 16)),
+                                             (3, 177, 1000, (-2, 5, 4))])
+def test_gemm_skinny_silu_epilogue(m, inter, k, shape):
     """Rows of w alternate gate and up rows; the product comes out as silu(gate) * up."""
     x = randn(m, k, dtype=torch.bfloat16, seed=32, scale=0.7)
     wg = randn(inter, k, dtype=torch.bfloat16, seed=33, scale=0.3)
     wu = randn(inter, k, dtype=torch.bfloat16, seed=34, scale=0.3)
     w = torch.stack([wg, wu], dim=1).reshape(2 * inter, k).contiguous()
-    out = K().gemm_skinny(x, w, torch.bfloat16, silu_pairs=True)
+    out = K().gemm_skinny(x, w, torch.bfloat16, silu_pairs=True, block_shape=shape)
     assert out.shape == (m, inter)
     ref = torch.nn.functional.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
     torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=2e-2 * math.sqrt(k) / 4)
