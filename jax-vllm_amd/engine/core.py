@@ -36,6 +36,16 @@ def _bucket(n: int, floor: int = 1) -> int:
     return b
 
 
+def _batch_bucket(n: int) -> int:
+    """Rows of the captured decode step that serves n requests: powers of two up to 16 (a step's
+    time hardly depends on the rows there), beyond that also the values half-way (24, 48, 96, ...):
+    at most a third of the rows are padding."""
+    b = _bucket(n)
+    if b > 16 and n <= b // 4 * 3:
+        return b // 4 * 3
+    return b
+
+
 class _DecodeGraph:
     """Fixed host and device buffers of one captured decode step and the graph itself."""
 
@@ -160,7 +170,7 @@ class EngineCore:
         rows added to reach the bucket size read the null page and store nothing."""
         cache, ps = self.cache, self.page_size
         r = len(entries)
-        rb = _bucket(r)
+        rb = _batch_bucket(r)
         n_groups = len(self.group_keys)
         widths = tuple(_bucket(max(len(cache.block_table(e.request_id, g)) for e in entries), 8)
                        for g in range(n_groups))
