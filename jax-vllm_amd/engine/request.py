@@ -61,5 +61,6 @@ class EngineStats:
     cache_hit_tokens: int = 0
     preemptions: int = 0
     stalled_portions: int = 0         # portions shortened or postponed for lack of pages
+    prefix_waits: int = 0             # admissions put off until a running request had computed shared pages
     max_batched_tokens: int = 0
     graph_replays: int = 0

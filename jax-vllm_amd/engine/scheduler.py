@@ -2,7 +2,8 @@
 budget, decodes, finishes and frees, and decides what happens when pages run out.
 
 Reference: ``jllm/engine/engine.py:161-168, 282-512``.  Kept: FIFO admission into at most
-``max_num_seqs`` slots, prefix-cache lookup at admission, a request's first token comes from
+``max_num_seqs`` slots (a request that would share pages which a running request is still
+computing waits for them and lets the ones behind it pass), prefix-cache lookup at admission, a request's first token comes from
 the step that ends its prompt, finish on ``max_new_tokens`` or on an emitted ``eos_id``,
 release at finish.  Changed: one mixed batch per step under ``max_num_batched_tokens``
 (decode tokens first, then prompt portions of any length) instead of one block per
@@ -129,11 +130,17 @@ class Scheduler:
                 out.items.append(ScheduledItem(req, n, n == req.num_remaining))
                 budget -= n
 
-        # 3. admission, FIFO
-        while self.waiting and budget > 0 and len(self.running) < cfg.max_num_seqs:
-            req = self.waiting[0]
+        # 3. admission, FIFO; a request whose leading pages a running request is about to compute
+        #    waits until they are there (it then takes them over instead of computing them again)
+        at = 0
+        while at < len(self.waiting) and budget > 0 and len(self.running) < cfg.max_num_seqs:
+            req = self.waiting[at]
             if req.arrival_step > self.step_index or req in out.preempted:
                 break
+            if self._waits_for_prefix(req):
+                self.stats.prefix_waits += 1
+                at += 1
+                continue
             tokens = req.all_tokens
             cached = cache.start(req.request_id, tokens)
             n = min(len(tokens) - cached, cfg.chunk_limit, budget)
@@ -143,7 +150,7 @@ class Scheduler:
                 if n <= 0:
                     cache.finish(req.request_id)     # gives the hit pages back untouched
                     break
-            self.waiting.popleft()
+            del self.waiting[at]
             req.num_computed = cached
             req.slot = cache.slot(req.request_id)
             req.admitted_order = self._admissions
@@ -163,6 +170,30 @@ class Scheduler:
 
         self.step_index += 1
         return out
+
+    def _waits_for_prefix(self, req: Request) -> bool:
+        """Whether a running request is still computing full pages whose tokens are the leading
+        tokens of ``req`` too (pages are found by their content once they are full)."""
+        if not getattr(self.cache, "prefix_cache", False):
+            return False
+        ps = self.config.page_size
+        tokens = req.all_tokens
+        limit = (len(tokens) - 1) // ps            # the page of the last token is never taken over
+        if limit == 0:
+            return False
+        first = tokens[:ps]
+        for other in self.running:
+            if other.num_remaining <= 1:
+                continue
+            theirs = other.all_tokens
+            if theirs[:ps] != first:
+                continue
+            n = 1
+            while n < limit and len(theirs) >= (n + 1) * ps and theirs[n * ps:(n + 1) * ps] == tokens[n * ps:(n + 1) * ps]:
+                n += 1
+            if other.num_computed < n * ps:
+                return True
+        return False
 
     def _arrived(self) -> bool:
         return bool(self.waiting) and self.waiting[0].arrival_step <= self.step_index

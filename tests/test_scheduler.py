@@ -159,6 +159,33 @@ def test_prefix_cache_decisions():
     assert core.steps[-1][0][1] == 48 and again == [expected(prompt + long[:17], 1)]
 
 
+def test_a_request_waits_for_pages_that_a_running_request_is_computing():
+    """Four prompts arrive together; two share their first 64 tokens.  The second of the two is
+    put off until the first has computed the shared pages, takes them over, and the ones behind it
+    are admitted meanwhile.  Tokens are what they are without the prefix cache."""
+    kw = dict(block_size=16, max_num_seqs=4, max_model_len=256, max_num_batched_tokens=96, max_chunk=32)
+    shared = list(range(64))
+    prompts = [shared + [70 + i for i in range(20)], shared + [80] * 9, [5] * 40, [6] * 33]
+    eng, core = make(**kw)
+    got = eng.generate(prompts, SamplingParams(max_new_tokens=3))
+    assert got == [expected(p, 3) for p in prompts]
+    first_step = {rid: i for i, log in reversed(list(enumerate(core.steps))) for rid, *_ in log}
+    ids = sorted(first_step)                                   # request ids in order of arrival
+    assert first_step[ids[0]] == 0 and first_step[ids[2]] == 0 and first_step[ids[3]] == 0
+    assert first_step[ids[1]] == 2                             # after two 32-token portions of the first
+    start = [log for log in core.steps[2] if log[0] == ids[1]][0]
+    assert start[1] == 64                                      # it begins behind the pages it took over
+    assert eng.stats.cache_hit_blocks == 4 and eng.stats.prefix_waits == 2
+    plain, _ = make(enable_prefix_cache=False, **kw)
+    assert plain.generate(prompts, SamplingParams(max_new_tokens=3)) == got
+    assert plain.stats.prefix_waits == 0 and plain.stats.cache_hit_blocks == 0
+    # the sharer does not wait for a request that has its prompt behind it already
+    eng2, _ = make(**kw)
+    eng2.generate([prompts[0]], SamplingParams(max_new_tokens=1))
+    eng2.generate([prompts[1]], SamplingParams(max_new_tokens=1))
+    assert eng2.stats.prefix_waits == 0 and eng2.stats.cache_hit_blocks == 4
+
+
 def test_requests_that_can_never_fit_are_refused():
     eng, _ = make(block_size=4, max_num_seqs=2, max_model_len=64, max_prefill_len=32, num_blocks=1 + 5)
     with pytest.raises(ValueError, match="empty prompt"):
@@ -227,8 +254,9 @@ def test_baseline_workload_b_under_a_24_token_budget():
     assert all(sum(n for _, _, n, _ in s) <= 24 for s in core.steps)
     mixed = [s for s in core.steps if any(n > 1 for _, _, n, _ in s) and any(n == 1 and c > 0 for _, c, n, _ in s)]
     assert mixed, "prompt portions never ran beside decoded tokens"
-    # the second sharer arrives one step after the first: only the first common page is full by then
-    assert eng.stats.cache_hit_blocks == 1
+    # the second sharer arrives one step after the first, when only the first common page is full:
+    # it waits one step for the second and takes both over
+    assert eng.stats.cache_hit_blocks == 2 and eng.stats.prefix_waits == 1
 
 
 @pytest.mark.parametrize("seed", range(4))
