@@ -479,6 +479,7 @@ extern "C" int jv_attn_prefill_groups_per_item() { return RT; }
 
 // ------------------------------------------------------------------------------------ decode
 constexpr int BND = 32;  // keys per wave iteration
+constexpr int DEC_TBL_MAX = 4096;  // page-table entries of a request that a decode block keeps in LDS
 
 __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(AttnArgs p) {
   extern __shared__ float smem[];  // per wave: m[16], l[16], acc[16][D]
@@ -488,15 +489,26 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
   const PageSplit ps{P, p.page_shift};
   const int mt_per_head = (G + 15) / 16;
   const int w = blockIdx.x;
-  const int r = p.work[w];
+  // Without a work list the requests are 0, 1, ... and request r's token is row r (a step of
+  // decoded tokens only): nothing has to be looked up before the loads below can start.  The
+  // kernel's time at small batches is its chain of dependent memory round trips (~1.5 us each
+  // for data the previous kernel wrote), so the request's page table row is copied to LDS at
+  // once, beside the load of its context length, instead of being read key range by key range
+  // after it.
+  const int r = p.work ? p.work[w] : w;
   const int g = blockIdx.y / mt_per_head, mt = blockIdx.y - g * mt_per_head;
   const int split = blockIdx.z;
-  const int tok = p.cu_seqlens[r];
+  const int* gtable = p.block_tables + (long long)r * p.table_stride;
+  int* tbl = (int*)(smem + 4 * (32 + 16 * D));
+  const bool table_in_lds = p.table_stride <= DEC_TBL_MAX;
+  if (table_in_lds)
+    for (int i = tid; i < p.table_stride; i += 256) tbl[i] = gtable[i];
+  const int tok = p.cu_seqlens ? p.cu_seqlens[r] : r;
   const int pos = p.context_lens[r];      // the query's position; keys 0..pos are stored
   const int kv_len = pos + 1;
   int kv_begin = 0;
   if (p.window > 0 && pos - p.window + 1 > 0) kv_begin = pos - p.window + 1;
-  const int* table = p.block_tables + (long long)r * p.table_stride;
+  auto page_at = [&](int idx) -> long long { return table_in_lds ? tbl[idx] : gtable[idx]; };
 
   const int hg = mt * 16 + li;
   const bool row_ok = hg < G;
@@ -523,6 +535,7 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  __syncthreads();   // the table row is in LDS
   // One tile's operands, global -> registers.  Nothing here looks at a loaded value, so a tile's
   // loads are in flight while the tile before it is multiplied.  Keys at or past kv_len read the
   // null page: their scores are masked by position, their V entries are zeroed before use.
@@ -534,7 +547,7 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
     for (int kt = 0; kt < 2; ++kt) {
       const int j = j0 + kt * 16 + li;
       const bool ok = j < kv_len;
-      const long long page = ok ? table[ps.index(j)] : 0;
+      const long long page = ok ? page_at(ps.index(j)) : 0;
       const bf16_t* krow = p.k_pages + ((page * p.nkv + g) * P + (ok ? ps.slot(j) : 0)) * (long long)D;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
@@ -546,7 +559,7 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
     for (int kt = 0; kt < 2; ++kt) {
       const int j = j0 + kt * 16 + lc * 4;
       const bool ok = j < kv_len;
-      const long long page = ok ? table[ps.index(j)] : 0;
+      const long long page = ok ? page_at(ps.index(j)) : 0;
       const bf16_t* vbase = p.v_pages + (page * p.nkv + g) * (long long)D * P + (ok ? ps.slot(j) : 0);
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) vf[kt][dt] = *(const bf16x4*)(vbase + (long long)(dt * 16 + li) * P);
@@ -677,8 +690,8 @@ __global__ void attn_decode_merge_kernel(AttnArgs p) {
   // All loads of a batch of 8 splits are issued before anything is computed from them: this
   // kernel's time is its chain of dependent memory round trips, not its arithmetic.
   const int w = blockIdx.x, head = blockIdx.y, d = threadIdx.x < D ? threadIdx.x : D - 1;
-  const int r = p.work[w];
-  const int tok = p.cu_seqlens[r];
+  const int r = p.work ? p.work[w] : w;
+  const int tok = p.cu_seqlens ? p.cu_seqlens[r] : r;
   const long long base = ((long long)w * p.nq + head) * p.num_splits;
   const float2* ml = (const float2*)p.part_ml + base;      // (max, sum) per split
   const float* pa = p.part_acc + base * D + d;
@@ -773,7 +786,8 @@ extern "C" int jv_attn_decode(void* out, const void* q, long long q_row_stride, 
   }
   const int G = nq / nkv, mt_per_head = (G + 15) / 16;
   if ((long long)nkv * mt_per_head > 65535 || a.num_splits > 65535) return (int)hipErrorInvalidValue;
-  const size_t shmem = 4 * (32 + 16 * D) * sizeof(float);
+  const size_t shmem = 4 * (32 + 16 * D) * sizeof(float) +
+                       (table_stride <= DEC_TBL_MAX ? (size_t)table_stride * sizeof(int) : 0);
   if (shmem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)attn_decode_kernel,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);

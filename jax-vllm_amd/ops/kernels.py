@@ -471,7 +471,8 @@ def _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlen
     _need(block_tables.dim() == 2, "block_tables must be [requests, pages]")
     for t, name in ((block_tables, "block_tables"), (cu_seqlens, "cu_seqlens"), (context_lens, "context_lens"),
                     (work, "work")):
-        _i32(t, name)
+        if t is not None:
+            _i32(t, name)
     _need(cu_seqlens.numel() == context_lens.numel() + 1 == block_tables.shape[0] + 1,
           "cu_seqlens, context_lens and block_tables disagree on the number of requests")
     return page_size
@@ -503,12 +504,16 @@ def attn_decode_scratch_floats(n_work: int, nq: int, num_splits: int, head_dim: 
 def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work, n_work,
                      nq, nkv, head_dim, scale, window=0, num_splits=1, scratch=None) -> None:
     """Attention of single decoded tokens.  ``work`` is int32 [n_work]: indices of the requests
-    (each with exactly one token in this step).  With ``num_splits`` > 1 a request's keys are
-    shared out to that many blocks and ``scratch`` (float32, ``attn_decode_scratch_floats``
-    entries) holds their partial results."""
+    (each with exactly one token in this step); None: the step holds decoded tokens only, request
+    r = 0 .. n_work-1 has its token in row r (the kernel then has nothing to look up before its
+    loads start).  With ``num_splits`` > 1 a request's keys are shared out to that many blocks and
+    ``scratch`` (float32, ``attn_decode_scratch_floats`` entries) holds their partial results."""
     page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
                              nq, nkv, head_dim)
-    _need(work.numel() >= n_work, "work list shorter than n_work")
+    if work is None:
+        _need(n_work == context_lens.numel() == out.shape[0], "without a work list every request has one token")
+    else:
+        _need(work.numel() >= n_work, "work list shorter than n_work")
     if num_splits > 1:
         _need(scratch is not None and scratch.is_cuda and scratch.dtype == torch.float32
               and scratch.numel() >= attn_decode_scratch_floats(n_work, nq, num_splits, head_dim),
@@ -516,7 +521,8 @@ def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_se
     lib = library.attention(head_dim)
     _check(
         lib.jv_attn_decode(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages),
-                           _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens),
+                           _ptr(block_tables), c_int(block_tables.shape[1]),
+                           _ptr(cu_seqlens if work is not None else None), _ptr(context_lens),
                            _ptr(work), c_int(n_work), c_int(page_size), c_int(nq), c_int(nkv), c_float(scale),
                            c_int(window or 0), c_int(num_splits), _ptr(scratch if num_splits > 1 else None),
                            _stream()),

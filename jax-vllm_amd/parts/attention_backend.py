@@ -27,7 +27,7 @@ BALANCE_BLOCKS = 768         # up to here prefill work items pair light row grou
 class MfmaPlan:
     prefill_work: Optional[torch.Tensor]   # int32 [n, 3]
     n_prefill: int
-    decode_work: Optional[torch.Tensor]    # int32 [n]
+    decode_work: Optional[torch.Tensor]    # int32 [n]; None when the step holds decoded tokens only
     n_decode: int
     num_splits: int
     scratch: Optional[torch.Tensor]
@@ -91,15 +91,16 @@ def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> Mfm
     decode = [r for r, ql in enumerate(ctx.q_lens_host) if ql == 1]
     max_kv_decode = max([ctx.context_lens_host[r] + 1 for r in decode], default=1)
     splits = decode_splits(len(decode), nkv * (-(-g // 16)), max_kv_decode) if decode else 1
-    flat = [x for item in prefill for x in item] + decode
+    decode_only = len(decode) == len(ctx.q_lens_host)       # requests 0, 1, ...: the kernel needs no list
+    flat = [x for item in prefill for x in item] + ([] if decode_only else decode)
     dev = torch.tensor(flat, dtype=torch.int32).pin_memory().to(device, non_blocking=True) if flat else None
     n_pre = len(prefill)
     scratch = None
     if decode and splits > 1:
         scratch = torch.empty(K.attn_decode_scratch_floats(len(decode), nq, splits, head_dim),
                               dtype=torch.float32, device=device)
-    return MfmaPlan(dev[: 3 * n_pre] if n_pre else None, n_pre, dev[3 * n_pre:] if decode else None, len(decode),
-                    splits, scratch)
+    return MfmaPlan(dev[: 3 * n_pre] if n_pre else None, n_pre,
+                    dev[3 * n_pre:] if decode and not decode_only else None, len(decode), splits, scratch)
 
 
 def run(att, out, qkv, ctx, mem) -> None:

@@ -477,6 +477,11 @@ def test_mfma_decode_attention(case, splits):
                          window or 0, splits, scratch)
     ref = _mfma_reference(qs, ks, vs, reqs, scale, window, nq, d)
     torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
+    # a step of decoded tokens only needs no work list: request r's token is row r
+    again = torch.full((dev["n"], nq * d), float("nan"), dtype=torch.bfloat16).cuda()
+    K().attn_decode_mfma(again, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                         dev["ctx"], None, len(order), nq, nkv, d, scale, window or 0, splits, scratch)
+    assert torch.equal(again, out)
 
 
 @pytest.mark.parametrize("far_key", [0, 15, 16, 31, 32, 63, 64, 255, 256, 511, 640])
