@@ -183,6 +183,67 @@ def test_qk_norm_rope_write(dtype, nq, nkv, d, rotary_dim, interleaved, with_nor
     torch.testing.assert_close(qkv2.float().view(t, nq + 2 * nkv, d)[:, :nq], got_q, rtol=0, atol=0)
 
 
+def _slot_pattern(kind: str, t: int, page_size: int):
+    base = 2 * page_size
+    if kind == "prompt":            # one prompt from the start of a page: every 8 tokens are one aligned run
+        return [base + i for i in range(t)]
+    if kind == "offset":            # a portion that starts in the middle of a page: no aligned run at all
+        return [base + 3 + i for i in range(t)]
+    if kind == "two_requests":      # a boundary between requests inside a group of 8, the second one unaligned
+        first = 130
+        second_base = base + 40 * page_size + 5
+        return [base + i for i in range(first)] + [second_base + i for i in range(t - first)]
+    g = torch.Generator().manual_seed(t + page_size)
+    slots = (torch.randperm(t + 64, generator=g)[:t] + base).tolist()
+    for i in (7, 8, 100, t - 1):
+        slots[i] = -1
+    return slots
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("page_size", [8, 16, 64])
+@pytest.mark.parametrize("kind", ["prompt", "offset", "two_requests", "scattered"])
+@pytest.mark.parametrize("nq,nkv,d,t", [(4, 2, 128, 300), (2, 3, 80, 259), (5, 3, 64, 270), (3, 1, 256, 257)])
+def test_values_of_many_tokens_reach_their_pages(dtype, page_size, kind, nq, nkv, d, t):
+    """From 256 tokens on the v heads go to their transposed pages 8 tokens at a time where 8
+    consecutive tokens have 8 consecutive, aligned slots, and one by one elsewhere, and q and k of
+    fully rotated heads of 64, 128 or 256 are prepared 16 bytes a lane: all must give what the
+    token-by-token path gives (the same call on portions below 256 tokens), v as an untouched copy."""
+    eps = 1e-6
+    slot_list = _slot_pattern(kind, t, page_size)
+    pages = max(slot_list) // page_size + 2
+    qkv = randn(t, (nq + 2 * nkv) * d, dtype=dtype, seed=31)
+    slots = torch.tensor(slot_list, dtype=torch.int32).cuda()
+    pos = torch.arange(t, dtype=torch.int32).cuda()
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, d, 2, dtype=torch.float32) / d))).cuda()
+    table = K().rope_table(pos, inv_freq)
+    qw, kw = 1 + 0.1 * randn(d, seed=32), 1 + 0.1 * randn(d, seed=33)
+
+    def run(portions):
+        x = qkv.clone()
+        kp = torch.zeros(pages, nkv, page_size, d, dtype=dtype).cuda()
+        vp = torch.zeros(pages, nkv, d, page_size, dtype=dtype).cuda()
+        for a, b in portions:
+            part = x[a:b].contiguous()
+            K().qk_norm_rope_write(part, slots[a:b].contiguous(), qw, kw, eps, table[a:b].contiguous(), d, False,
+                                   kp, vp, page_size, nq, nkv, d)
+            x[a:b] = part
+        return x, kp, vp
+
+    whole = run([(0, t)])
+    pieces = run([(0, 101), (101, 250), (250, t)])
+    # q and k: the two paths add the squares of a head in different orders
+    torch.testing.assert_close(whole[0].float(), pieces[0].float(), **tol(dtype, f32=2e-5, bf16=2e-2))
+    torch.testing.assert_close(whole[1].float(), pieces[1].float(), **tol(dtype, f32=2e-5, bf16=2e-2))
+    torch.testing.assert_close(whole[2], pieces[2], rtol=0, atol=0)
+    exp_v = torch.zeros(pages, nkv, d, page_size, dtype=dtype).cuda()
+    v = qkv.view(t, nq + 2 * nkv, d)[:, nq + nkv:]
+    for i, s_ in enumerate(slot_list):
+        if s_ >= 0:
+            exp_v[s_ // page_size, :, :, s_ % page_size] = v[i]
+    torch.testing.assert_close(whole[2], exp_v, rtol=0, atol=0)
+
+
 @pytest.mark.parametrize("nq,nkv,d,n_parts,t,with_norm", [(6, 2, 128, 2, 5, True), (4, 4, 256, 4, 16, True),
                                                          (32, 8, 128, 4, 8, True), (3, 1, 128, 3, 9, False)])
 def test_qk_norm_rope_write_from_partial_products(nq, nkv, d, n_parts, t, with_norm):
