@@ -1,7 +1,7 @@
 """Measurement of the engine on one MI355X: decode tokens/s at batch 8 (the headline), with
 prefill tokens/s at 2,048 tokens and decode at batch 1 and 64 beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|14b|32b]
 
 The model has the layer sizes of BASELINE.json ``configs[2]`` (Qwen3-8B shape) with random
 weights drawn on the device; prompts are seeded uniform-random token ids of 1,024 tokens;
@@ -29,6 +29,14 @@ QWEN3_8B = dict(
     num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
     rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960,
 )
+# the other shapes of BASELINE.json (configs[3] and [4]), for runs at further sizes: --shape
+SHAPES = {
+    "8b": ("Qwen3-8B-shaped", QWEN3_8B),
+    "14b": ("Qwen3-14B-shaped", dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40,
+                                     intermediate_size=17408)),
+    "32b": ("Qwen3-32B-shaped", dict(QWEN3_8B, num_hidden_layers=64, hidden_size=5120, num_attention_heads=64,
+                                     intermediate_size=25600)),
+}
 PROMPT_LEN = 1024
 MAX_CONTEXT = 8192
 PREFILL_TOKENS = 2048
@@ -97,8 +105,10 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--layers", type=int, default=QWEN3_8B["num_hidden_layers"],
-                    help="run only the first layers of the 36 (reported in config)")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+                    help="layer sizes: 8b is the headline configuration, the others are for runs at further sizes")
+    ap.add_argument("--layers", type=int, default=None,
+                    help="run only the first layers of the shape's (both numbers are reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="measure the headline batch only")
     ap.add_argument("--only", choices=["prefill", "decode"], default=None,
@@ -116,8 +126,9 @@ def main():
 
     from jax_vllm_amd import LLM
 
-    cfg = dict(QWEN3_8B)
-    layers = args.layers
+    model_name, shape = SHAPES[args.shape]
+    cfg = dict(shape)
+    layers = args.layers if args.layers is not None else shape["num_hidden_layers"]
     cfg["num_hidden_layers"] = layers
     vocab = cfg["vocab_size"]
     rng = np.random.default_rng(0)
@@ -165,7 +176,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
         "data": "synthetic: seeded uniform-random token ids, random-init weights N(0,0.02), norms 1+N(0,0.02)",
         "config": {
-            "model": "Qwen3-8B-shaped", "layers": layers, "layers_full": QWEN3_8B["num_hidden_layers"],
+            "model": model_name, "layers": layers, "layers_full": shape["num_hidden_layers"],
             "hidden": cfg["hidden_size"], "q_heads": nq, "kv_heads": cfg["num_key_value_heads"], "head_dim": d,
             "intermediate": cfg["intermediate_size"], "vocab": vocab, "global_batch": args.batch,
             "seq_len": PROMPT_LEN, "max_context": MAX_CONTEXT, "mean_decode_context": round(mean_ctx, 1),

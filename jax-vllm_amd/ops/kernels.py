@@ -332,6 +332,43 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     return out
 
 
+def gemm_tile64(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_pairs: bool = False,
+                ksplit: int = 1, out=None) -> torch.Tensor:
+    """x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w [N, K] with blocks that take 64
+    rows of w against all rows of x: the weight-streaming product of decode steps with 17..64
+    requests where the library is slow (narrow outputs over a long inner size).  ``silu_pairs`` and ``ksplit`` as in ``gemm_skinny``:
+    silu(x.w[2j]) * (x.w[2j+1]) as bfloat16 [M, N/2], or float32 partial products [ksplit, M, N] to
+    be added in order (every group needs at least one round of 256 columns)."""
+    _dev(x, w, out)
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_tile64 takes bfloat16")
+    m = x.shape[0]
+    n, k = w.shape
+    _need(x.dim() == 2 and x.shape[1] == k, "inner sizes differ")
+    _need(m <= SKINNY_MAX_ROWS, f"gemm_tile64 takes at most {SKINNY_MAX_ROWS} rows")
+    _need(k % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0,
+          "the inner size and the row stride must be multiples of 8")
+    _need(w.is_contiguous(), "w must be contiguous")
+    _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
+    _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and ksplit == 1),
+          "the silu epilogue writes bfloat16, needs an even number of rows of w and an inner size in one piece")
+    rounds = -(-k // 256)
+    _need(ksplit >= 1 and (ksplit == 1 or (out_dtype == torch.float32 and -(-rounds // ksplit) * (ksplit - 1) < rounds)),
+          "sharing the inner size out needs float32 output and a round of 256 columns for every group")
+    n_out = n // 2 if silu_pairs else n
+    shape = (m, n_out) if ksplit == 1 else (ksplit, m, n_out)
+    if out is None:
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    _need(out.shape == shape and out.dtype == out_dtype and out.is_contiguous(),
+          "out must be [M, N] (or [M, N/2], or [ksplit, M, N]) of the output type")
+    _check(
+        library.core().jv_gemm_tile64_bf16(
+            _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.stride(0)), c_longlong(n_out),
+            c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_pairs else 0), c_int(ksplit), _stream()),
+        "gemm_tile64",
+    )
+    return out
+
+
 _cu_count = {}
 
 
@@ -351,33 +388,53 @@ def _stay_pieces(k: int, parts: int):
     return None
 
 
+TILE64 = (-3, 0, 0)                 # block shape that stands for ``gemm_tile64`` in a plan
+TILE64_MIN_SHARE = 3072             # columns a block of gemm_tile64 needs to pay for its start
+LIBRARY_MAX_INNER = 12288           # beyond this inner size the library's choice for few rows collapses
+
+
 def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok: bool = False, device=None):
-    """How ``linear`` runs a bfloat16 product at few rows: (block_shape, ksplit) for ``gemm_skinny``,
-    or None for the library.  All thresholds are measured on MI355X at the matrix shapes of an
-    8B-class model (pure reads of the same bytes: 33 MB 6.5 us, 50 MB 9.1, 101 MB 16.5, 201 MB 33.5).
+    """How ``linear`` runs a bfloat16 product at few rows: (block_shape, ksplit) for ``gemm_skinny``
+    (``TILE64`` as block shape: for ``gemm_tile64``), or None for the library.  All thresholds are
+    measured on MI355X at the matrix shapes of 8B-, 14B- and 32B-class models (pure reads of the
+    same bytes: 33 MB 6.5 us, 50 MB 9.1, 101 MB 16.5, 201 MB 33.5).
 
     * wide matrices (>= 1,024 row tiles), inner size <= 4,096, 3..16 rows: blocks that stay, one per
       compute unit (two for very wide ones), x in registers: 201 MB in 38 us at 8 rows and 40.5 at
       16, against 42 and 53 with x staged per block, 44 by the library;
-    * narrow matrices whose reader adds partial products: the inner size shared out to 4 groups so
-      that ~1,000 blocks stream (33 MB: 8.6 us against 11.0 from 256 blocks);
+    * narrow matrices whose reader adds partial products, up to 16 rows: the inner size shared out
+      to 4 groups so that ~1,000 blocks stream (33 MB: 8.6 us against 11.0 from 256 blocks); staying
+      blocks at inner sizes up to 4,096, x resident in LDS beyond;
+    * the same at 17..64 rows when every block gets at least 3,072 columns: blocks of 64 rows of w,
+      one per compute unit (the feed-forward's second product: 4,096 x 12,288 at 64 rows 30 us
+      against the library's 37; 5,120 x 17,408 65 against 131; 5,120 x 25,600 91 against 157);
     * one or two rows against wide matrices: x resident in LDS (chosen inside the kernel library);
-    * 9..16 rows of a large matrix that fits none of these: the library (its wider tiles amortise x);
+    * 9..16 rows of a large matrix that fits none of these: the library (its wider tiles amortise
+      x), unless the inner size is beyond 12,288, where the library needs 113 us for the 178 MB
+      that x resident in LDS streams in 45;
     * otherwise x staged chunk by chunk in LDS.
     """
-    if m > SKINNY_AUTO_ROWS or k % 8:
+    if k % 8:
+        return None
+    cus = _compute_units(device) if device is not None else 256
+    narrow = partial_ok and not silu_pairs and n % 4 == 0 and n <= PARTIAL_SUM_MAX_WIDTH
+    if m > SKINNY_AUTO_ROWS:
+        if narrow and m <= SKINNY_MAX_ROWS:
+            parts = min(4, cus // -(-n // 64))
+            rounds = -(-k // 256)
+            if parts >= 2 and k >= parts * TILE64_MIN_SHARE and -(-rounds // parts) * (parts - 1) < rounds:
+                return TILE64, parts
         return None
     tiles = -(-n // 16)
-    cus = _compute_units(device) if device is not None else 256
-    if partial_ok and not silu_pairs and n % 4 == 0 and n <= PARTIAL_SUM_MAX_WIDTH and tiles * 2 <= PARTIAL_BLOCKS:
+    if narrow and tiles * 2 <= PARTIAL_BLOCKS:
         parts = min(4, -(-PARTIAL_BLOCKS // tiles))
         parts = 4 if parts == 3 else parts
         if parts > 1:
-            nl = _stay_pieces(k, parts)
+            nl = _stay_pieces(k, parts) if k <= 4096 else None
             if nl is not None:
                 return (-2, 2 * cus, nl), parts
             phases = -(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32))
-            if phases >= parts and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX):
+            if phases >= parts and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX and k <= LIBRARY_MAX_INNER):
                 return PARTIAL_SHAPE, parts
     if m >= 3 and tiles >= 4 * cus:
         nl = _stay_pieces(k, 1)
@@ -392,10 +449,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
     """x @ w.T for w stored [out, in].
 
     float32: the library's own float-FMA kernel (no reduced-precision matrix mode).
-    bfloat16, at most 16 rows: a weight-streaming MFMA kernel of this library (``streaming_plan``).
-    bfloat16, more rows: a plain library matrix product (hipBLASLt through torch), float accumulation.
+    bfloat16, at most 16 rows (and some shapes up to 64): a weight-streaming MFMA kernel of this
+    library (``streaming_plan``).
+    bfloat16 otherwise: a plain library matrix product (hipBLASLt through torch), float accumulation.
     With ``partial_ok`` the caller takes a float32 stack [parts, M, N] of partial products as well
-    (to be added in order, as ``add_rmsnorm`` does); it is returned for narrow matrices at few rows.
+    (to be added in order, as ``add_rmsnorm`` does); it is returned for narrow matrices at up to 64 rows.
     With ``silu_pairs`` the rows of w alternate gate and up rows and the result is
     silu(x.w[2j]) * (x.w[2j+1]) of width N/2 (an epilogue of the streaming kernels, a kernel of
     its own after the library's product).
@@ -408,6 +466,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
                               partial_ok and out_dtype in (None, torch.bfloat16), x.device)
         if plan is not None:
             shape, parts = plan
+            if shape == TILE64:
+                return gemm_tile64(x, w, torch.float32, ksplit=parts)
             if parts > 1:
                 return gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=parts)
             return gemm_skinny(x, w, out_dtype or torch.bfloat16, silu_pairs=silu_pairs, block_shape=shape)

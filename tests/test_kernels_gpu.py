@@ -722,6 +722,85 @@ def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
         K().gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=1000)   # more parts than phases
 
 
+TILE64_CASES = [(17, 64, 256, 1), (64, 128, 2048, 4), (33, 200, 1000, 2), (48, 72, 3080, 3), (64, 64, 264, 2),
+                (20, 4096, 12288, 4), (1, 130, 520, 1), (64, 5120, 17408, 3)]
+
+
+@pytest.mark.parametrize("m,n,k,ksplit", TILE64_CASES)
+def test_gemm_tile64(m, n, k, ksplit):
+    """Blocks of 64 rows of w against up to 64 rows of x: whole products and partial products of a
+    shared-out inner size, at sizes that end inside a tile of w, inside a row tile of x, inside a
+    chunk of 256 columns and inside a 32-column step; rows of x and w beyond the sizes and columns
+    beyond a block's share must contribute nothing."""
+    x = randn(m, k, dtype=torch.bfloat16, seed=51, scale=0.5)
+    w = randn(n, k, dtype=torch.bfloat16, seed=52, scale=0.1)
+    ref = x.double() @ w.double().T
+    out_dtype = torch.float32 if ksplit > 1 else torch.bfloat16
+    y = K().gemm_tile64(x, w, out_dtype, ksplit=ksplit)
+    if ksplit > 1:
+        assert y.shape == (ksplit, m, n) and y.dtype == torch.float32
+        torch.testing.assert_close(y.sum(0).double(), ref, rtol=1e-3, atol=2e-3 * math.sqrt(k) / 8)
+        # every group holds its own columns only: group 0 equals the product over its share
+        share = -(-(-(-k // 256)) // ksplit) * 256
+        torch.testing.assert_close(y[0].double(), x[:, :share].double() @ w[:, :share].double().T,
+                                   rtol=1e-3, atol=2e-3 * math.sqrt(k) / 8)
+    else:
+        assert y.shape == (m, n) and y.dtype == torch.bfloat16
+        torch.testing.assert_close(y.double(), ref, rtol=2e-2, atol=2e-2 * math.sqrt(k) / 8)
+        yf = K().gemm_tile64(x, w, torch.float32)
+        torch.testing.assert_close(yf.double(), ref, rtol=1e-3, atol=2e-3 * math.sqrt(k) / 8)
+    # the same call again gives the same bits (fixed order of every sum)
+    torch.testing.assert_close(K().gemm_tile64(x, w, out_dtype, ksplit=ksplit), y, rtol=0, atol=0)
+
+
+def test_gemm_tile64_silu_epilogue_and_refusals():
+    x = randn(40, 1024, dtype=torch.bfloat16, seed=53, scale=0.5)
+    w = randn(300, 1024, dtype=torch.bfloat16, seed=54, scale=0.1)
+    g, u = w[0::2].double(), w[1::2].double()
+    want = torch.nn.functional.silu(x.double() @ g.T) * (x.double() @ u.T)
+    got = K().gemm_tile64(x, w, silu_pairs=True)
+    assert got.shape == (40, 150)
+    torch.testing.assert_close(got.double(), want, rtol=2e-2, atol=2e-2)
+    with pytest.raises(ValueError):
+        K().gemm_tile64(randn(65, 1024, dtype=torch.bfloat16), w)                    # more than 64 rows
+    with pytest.raises(ValueError):
+        K().gemm_tile64(x, w, torch.float32, ksplit=5)                              # 4 chunks of 256 for 5 groups
+    with pytest.raises(ValueError):
+        K().gemm_tile64(x, w, torch.bfloat16, ksplit=2)                             # partial products are float32
+    with pytest.raises(ValueError):
+        K().gemm_tile64(x, w, silu_pairs=True, ksplit=2, out_dtype=torch.float32)   # no activation of a partial sum
+
+
+def test_linear_takes_blocks_of_64_rows_for_a_long_inner_size():
+    """17..64 rows against a narrow matrix with a long inner size (the feed-forward's second product):
+    ``linear`` hands out partial products from ``gemm_tile64`` that ``add_rmsnorm`` adds; the same
+    product without a reader for partial sums is the library's."""
+    kern = K()
+    m, n, k = 40, 1024, 12288
+    x = randn(m, k, dtype=torch.bfloat16, seed=55, scale=0.5)
+    w = randn(n, k, dtype=torch.bfloat16, seed=56, scale=0.05)
+    plan = kern.streaming_plan(m, n, k, partial_ok=True, device=x.device)
+    assert plan == (kern.TILE64, 4)
+    assert kern.streaming_plan(m, n, k, partial_ok=False, device=x.device) is None
+    assert kern.streaming_plan(m, n, 4096, partial_ok=True, device=x.device) is None      # too few columns a block
+    assert kern.streaming_plan(12, 5120, 17408, partial_ok=True, device=x.device) == (kern.PARTIAL_SHAPE, 4)
+    parts = kern.linear(x, w, partial_ok=True)
+    assert parts.shape == (4, m, n) and parts.dtype == torch.float32
+    ref = x.double() @ w.double().T
+    torch.testing.assert_close(parts.sum(0).double(), ref, rtol=1e-3, atol=2e-2)
+    torch.testing.assert_close(kern.linear(x, w).double(), ref, rtol=2e-2, atol=2e-1)
+    # the reader: residual + ordered sum of the parts, then the norm
+    h = randn(m, n, seed=57)
+    weight = 1 + 0.1 * randn(n, seed=58)
+    h2 = h.clone()
+    out = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    kern.add_rmsnorm(h2, parts, weight, out, 1e-6)
+    want_h = h + ((parts[0] + parts[1]) + parts[2]) + parts[3]
+    torch.testing.assert_close(h2, want_h, rtol=1e-6, atol=1e-6)
+    want = want_h * torch.rsqrt((want_h * want_h).mean(-1, keepdim=True) + 1e-6) * weight
+    torch.testing.assert_close(out.float(), want, rtol=2e-2, atol=2e-2)
+
+
 def test_linear_follows_its_plan_and_all_roads_agree():
     """``linear`` at few rows: the staying blocks, the shared-out inner size, the staged chunks and
     the library must give the same numbers up to rounding, with and without the silu epilogue."""
