@@ -100,6 +100,41 @@ def measure_prefill(llm, rng, vocab, repeats=3):
     return best
 
 
+def measure_mixed(llm, rng, vocab, running=32, joining=4, join_len=3000, shared=1024):
+    """The continuous-batching mix of BASELINE.json configs[3]: ``running`` requests decode at contexts
+    uniform in [512, 4096] when ``joining`` prompts of ``join_len`` tokens arrive, two of which share
+    their first ``shared`` tokens; timed from their arrival until all of them have their first token."""
+    from jax_vllm_amd import SamplingParams
+
+    keep = SamplingParams(max_new_tokens=256)   # far more than the steps this takes
+    first = [llm.add_request(rng.integers(0, vocab, size=int(n)).tolist(), keep)
+             for n in rng.integers(512, 4097, size=running)]
+    while any(not llm.requests[r].output_ids for r in first):
+        llm.step()
+    for _ in range(8):                       # decode steps of the running requests alone (captured)
+        llm.step()
+    sync()
+    prefix = rng.integers(0, vocab, size=shared).tolist()
+    prompts = [rng.integers(0, vocab, size=join_len).tolist() for _ in range(joining)]
+    for p in prompts[-2:]:
+        p[:shared] = prefix
+    before = (llm.stats.prefill_tokens, llm.stats.decode_tokens, llm.stats.cache_hit_tokens)
+    t0 = time.perf_counter()
+    new = [llm.add_request(p, SamplingParams(max_new_tokens=64)) for p in prompts]
+    steps, longest, last = 0, 0.0, t0
+    while any(not llm.requests[r].output_ids for r in new):
+        llm.step()
+        sync()
+        now = time.perf_counter()
+        longest, last, steps = max(longest, now - last), now, steps + 1
+    dt = time.perf_counter() - t0
+    pre, dec, hit = (a - b for a, b in zip((llm.stats.prefill_tokens, llm.stats.decode_tokens,
+                                            llm.stats.cache_hit_tokens), before))
+    return {"mixed_tokens_per_s": round((pre + dec) / dt, 1), "steps": steps, "ms_per_step": round(dt / steps * 1e3, 3),
+            "longest_step_ms": round(longest * 1e3, 3), "prompt_tokens_computed": pre, "decoded_tokens": dec,
+            "cache_hit_tokens": hit, "running": running, "joining": joining}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -111,8 +146,9 @@ def main():
                     help="run only the first layers of the shape's (both numbers are reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="measure the headline batch only")
-    ap.add_argument("--only", choices=["prefill", "decode"], default=None,
-                    help="run one phase alone and print its result (for profiling)")
+    ap.add_argument("--only", choices=["prefill", "decode", "mixed"], default=None,
+                    help="run one phase alone and print its result (for profiling); mixed: 32 running decodes "
+                         "joined by 4 prompts of 3,000 tokens in portions of 512 under a budget of 2,048")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
                     help="with --only decode: prompt length of the decoding requests (long-context runs)")
@@ -134,6 +170,14 @@ def main():
     rng = np.random.default_rng(0)
     max_batch = args.batch if (args.skip_points or args.only) else max(64, args.batch)
     block = 16
+    if args.only == "mixed":
+        llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=36, max_model_len=8192,
+                  num_blocks=1 + 32 * (4608 // block) + 4 * (3200 // block), max_num_batched_tokens=2048,
+                  max_chunk=512, enable_prefix_cache=True)
+        res = measure_mixed(llm, rng, vocab)
+        res.update(model=model_name, layers=layers)
+        print(json.dumps(res), flush=True)
+        return
     llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=max_batch,
               max_model_len=max(MAX_CONTEXT, args.prompt_len + 2 * 1024),
               num_blocks=1 + max_batch * (-(-(args.prompt_len + 2 * 1024) // block)),
