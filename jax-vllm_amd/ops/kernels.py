@@ -510,6 +510,24 @@ def attn_prefill_geometry(head_dim: int) -> tuple[int, int]:
     return 64, (2 if head_dim <= 128 else 1)
 
 
+_checked_attention_libraries = set()
+
+
+def _attention_library(head_dim: int):
+    """The attention library of a head size; on its first use the numbers this module plans with
+    (rows of a group, groups per work item, scratch size) are compared with the library's own."""
+    lib = library.attention(head_dim)
+    if head_dim not in _checked_attention_libraries:
+        lib.jv_attn_decode_scratch_floats.restype = c_longlong
+        got = (lib.jv_attn_head_dim(), lib.jv_attn_prefill_group_rows(), lib.jv_attn_prefill_groups_per_item(),
+               lib.jv_attn_decode_scratch_floats(c_int(3), c_int(5), c_int(7)))
+        want = (head_dim, *attn_prefill_geometry(head_dim), attn_decode_scratch_floats(3, 5, 7, head_dim))
+        if got != want:
+            raise KernelArgumentError(f"attention library for head size {head_dim} reports {got}, the planner expects {want}")
+        _checked_attention_libraries.add(head_dim)
+    return lib
+
+
 def mfma_attention_supported(dtype, head_dim: int, page_size: int) -> bool:
     """The matrix-core kernels take bfloat16, head sizes that are multiples of 16 up to 256 and
     page sizes that are multiples of 8; everything else goes to the generic kernel."""
@@ -547,7 +565,7 @@ def attn_prefill_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_s
     page_size = _attn_common(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_seqlens, context_lens, work,
                              nq, nkv, head_dim)
     _need(work.numel() >= 3 * n_work, "work list shorter than n_work")
-    lib = library.attention(head_dim)
+    lib = _attention_library(head_dim)
     _check(
         lib.jv_attn_prefill(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages),
                             _ptr(block_tables), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens),
@@ -578,7 +596,7 @@ def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_se
         _need(scratch is not None and scratch.is_cuda and scratch.dtype == torch.float32
               and scratch.numel() >= attn_decode_scratch_floats(n_work, nq, num_splits, head_dim),
               "scratch too small for the splits")
-    lib = library.attention(head_dim)
+    lib = _attention_library(head_dim)
     _check(
         lib.jv_attn_decode(_ptr(out), _ptr(q), c_longlong(q_row_stride), _ptr(k_pages), _ptr(v_pages),
                            _ptr(block_tables), c_int(block_tables.shape[1]),
