@@ -418,7 +418,7 @@ static int launch_persistent(void* y, const void* x, const void* W, int M, int N
   return JV_LAUNCH_CHECK();
 }
 
-// wr == -2: nks = NL in {4, 8, 16}, wk = blocks in all; the inner size must be at most
+// wr == -2: nks = NL in {4, 5, 8, 10, 12, 16, 17}, wk = blocks in all; the inner size must be at most
 // ksplit * 8 * NL * 32 and more than (ksplit - 1) * 8 * NL * 32
 template <typename OutT, bool PAIRS>
 static int dispatch_persistent(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
@@ -428,8 +428,12 @@ static int dispatch_persistent(int nl, void* y, const void* x, const void* W, in
     return (int)hipErrorInvalidValue;
   switch (nl) {
     case 4: return launch_persistent<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 5: return launch_persistent<5, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
     case 8: return launch_persistent<8, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 10: return launch_persistent<10, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 12: return launch_persistent<12, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
     case 16: return launch_persistent<16, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 17: return launch_persistent<17, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
   }
   return (int)hipErrorInvalidValue;
 }

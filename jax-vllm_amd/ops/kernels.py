@@ -309,7 +309,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     _need(m <= SKINNY_MAX_ROWS, f"gemm_skinny takes at most {SKINNY_MAX_ROWS} rows")
     _need(k % 8 == 0, "the inner size must be a multiple of 8")
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
-    _need(block_shape[0] != -2 or (m <= 16 and block_shape[2] in (4, 8, 16)
+    _need(block_shape[0] != -2 or (m <= 16 and block_shape[2] in STAY_PIECES
                                    and 256 * block_shape[2] * (ksplit - 1) < k <= 256 * block_shape[2] * ksplit),
           "the organisation with blocks that stay takes at most 16 rows and an inner size of ksplit * 256 * pieces at most")
     _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
@@ -379,10 +379,13 @@ def _compute_units(device) -> int:
     return n
 
 
+STAY_PIECES = (4, 5, 8, 10, 12, 16, 17)   # weight pieces per wave the staying blocks are built for
+
+
 def _stay_pieces(k: int, parts: int):
-    """Weight pieces per wave (4, 8 or 16) with which ``parts`` groups of staying blocks cover an
-    inner size of k exactly (each group 8 waves x pieces x 32 columns), or None."""
-    for nl in (4, 8, 16):
+    """Weight pieces per wave with which ``parts`` groups of staying blocks cover an inner size
+    of k exactly (each group 8 waves x pieces x 32 columns), or None."""
+    for nl in STAY_PIECES:
         if 256 * nl * (parts - 1) < k <= 256 * nl * parts:
             return nl
     return None
@@ -404,7 +407,9 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
       16, against 42 and 53 with x staged per block, 44 by the library;
     * narrow matrices whose reader adds partial products, up to 16 rows: the inner size shared out
       to 4 groups so that ~1,000 blocks stream (33 MB: 8.6 us against 11.0 from 256 blocks); staying
-      blocks at inner sizes up to 4,096, x resident in LDS beyond;
+      blocks at inner sizes up to 4,096 and where a group's share is long (4,096 x 12,288 at 8 rows:
+      21.1 us against 24.9 with x resident in LDS, at 16 rows 22.1 against 30.4; 5,120 x 17,408:
+      36.4 against 40.8), x resident in LDS otherwise (5,120 x 8,192: 21.0 against 22.8);
     * the same at 17..64 rows when every block gets at least 3,072 columns: blocks of 64 rows of w,
       one per compute unit (the feed-forward's second product: 4,096 x 12,288 at 64 rows 30 us
       against the library's 37; 5,120 x 17,408 65 against 131; 5,120 x 25,600 91 against 157);
@@ -430,9 +435,10 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
         parts = min(4, -(-PARTIAL_BLOCKS // tiles))
         parts = 4 if parts == 3 else parts
         if parts > 1:
-            nl = _stay_pieces(k, parts) if k <= 4096 else None
-            if nl is not None:
-                return (-2, 2 * cus, nl), parts
+            nl = _stay_pieces(k, parts)
+            if nl is not None and (k <= 4096 or nl >= 12 or m > 8):
+                # up to 8 pieces two blocks fit a compute unit; beyond, one block each walks its tiles
+                return (-2, (2 if nl <= 8 else 1) * cus, nl), parts
             phases = -(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32))
             if phases >= parts and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX and k <= LIBRARY_MAX_INNER):
                 return PARTIAL_SHAPE, parts

@@ -783,7 +783,8 @@ def test_linear_takes_blocks_of_64_rows_for_a_long_inner_size():
     assert plan == (kern.TILE64, 4)
     assert kern.streaming_plan(m, n, k, partial_ok=False, device=x.device) is None
     assert kern.streaming_plan(m, n, 4096, partial_ok=True, device=x.device) is None      # too few columns a block
-    assert kern.streaming_plan(12, 5120, 17408, partial_ok=True, device=x.device) == (kern.PARTIAL_SHAPE, 4)
+    few = kern.streaming_plan(12, 5120, 17408, partial_ok=True, device=x.device)     # not the library's either
+    assert few is not None and few[1] == 4 and few[0][0] in (-1, -2)
     parts = kern.linear(x, w, partial_ok=True)
     assert parts.shape == (4, m, n) and parts.dtype == torch.float32
     ref = x.double() @ w.double().T
