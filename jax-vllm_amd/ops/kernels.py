@@ -49,6 +49,8 @@ def _dev(*tensors) -> None:
 
 
 def _check(code: int, name: str) -> None:
+    if code == 1:   # hipErrorInvalidValue: what an entry point returns for sizes it is not built for
+        raise KernelArgumentError(f"{name}: the kernel library refused these sizes or this block shape")
     if code != 0:
         raise RuntimeError(f"{name}: HIP error {code}")
 
@@ -382,6 +384,14 @@ def _compute_units(device) -> int:
 STAY_PIECES = (4, 5, 8, 10, 12, 16, 17)   # weight pieces per wave the staying blocks are built for
 
 
+def _fit_parts(units: int, parts: int) -> int:
+    """The most groups, at most ``parts``, among which ``units`` (phases, chunks) can be shared out
+    in equal whole shares without leaving a group empty."""
+    while parts > 1 and -(-units // parts) * (parts - 1) >= units:
+        parts -= 1
+    return parts
+
+
 def _stay_pieces(k: int, parts: int):
     """Weight pieces per wave with which ``parts`` groups of staying blocks cover an inner size
     of k exactly (each group 8 waves x pieces x 32 columns), or None."""
@@ -425,9 +435,8 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     narrow = partial_ok and not silu_pairs and n % 4 == 0 and n <= PARTIAL_SUM_MAX_WIDTH
     if m > SKINNY_AUTO_ROWS:
         if narrow and m <= SKINNY_MAX_ROWS:
-            parts = min(4, cus // -(-n // 64))
-            rounds = -(-k // 256)
-            if parts >= 2 and k >= parts * TILE64_MIN_SHARE and -(-rounds // parts) * (parts - 1) < rounds:
+            parts = _fit_parts(-(-k // 256), min(4, cus // -(-n // 64)))
+            if parts >= 2 and k >= parts * TILE64_MIN_SHARE:
                 return TILE64, parts
         return None
     tiles = -(-n // 16)
@@ -439,9 +448,9 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
             if nl is not None and (k <= 4096 or nl >= 12 or m > 8):
                 # up to 8 pieces two blocks fit a compute unit; beyond, one block each walks its tiles
                 return (-2, (2 if nl <= 8 else 1) * cus, nl), parts
-            phases = -(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32))
-            if phases >= parts and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX and k <= LIBRARY_MAX_INNER):
-                return PARTIAL_SHAPE, parts
+            fewer = _fit_parts(-(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32)), parts)
+            if fewer > 1 and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX and k <= LIBRARY_MAX_INNER):
+                return PARTIAL_SHAPE, fewer
     if m >= 3 and tiles >= 4 * cus:
         nl = _stay_pieces(k, 1)
         if nl is not None:

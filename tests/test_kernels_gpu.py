@@ -802,6 +802,28 @@ def test_linear_takes_blocks_of_64_rows_for_a_long_inner_size():
     torch.testing.assert_close(out.float(), want, rtol=2e-2, atol=2e-2)
 
 
+@pytest.mark.parametrize("k", [512, 1000, 1024, 2560, 3072, 5120, 6152, 12288])
+def test_linear_at_every_size_runs_a_plan_the_library_accepts(k):
+    """Whatever ``streaming_plan`` picks for a size must be a plan the kernels accept and must give
+    the product: rows 1..64, widths and inner sizes that are no powers of two, inner sizes that do
+    not share out evenly (3,072 = 6 phases for 4 groups), with and without a reader of partial
+    products, with and without the silu epilogue."""
+    kern = K()
+    for n in (64, 1000, 1024, 4104):
+        w = randn(n, k, dtype=torch.bfloat16, seed=n + k, scale=0.05)
+        for m in (1, 5, 8, 12, 16, 17, 40, 64):
+            x = randn(m, k, dtype=torch.bfloat16, seed=m, scale=0.5)
+            ref = x.double() @ w.double().T
+            tol_ = dict(rtol=2e-2, atol=2e-2 * math.sqrt(k) / 8)
+            y = kern.linear(x, w, partial_ok=True)
+            y = y.sum(0) if y.dim() == 3 else y
+            torch.testing.assert_close(y.double(), ref, **tol_)
+            torch.testing.assert_close(kern.linear(x, w).double(), ref, **tol_)
+            act = kern.linear(x, w, silu_pairs=True)
+            want = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
+            torch.testing.assert_close(act.double(), want, rtol=3e-2, atol=3e-2 * math.sqrt(k) / 8)
+
+
 def test_linear_follows_its_plan_and_all_roads_agree():
     """``linear`` at few rows: the staying blocks, the shared-out inner size, the staged chunks and
     the library must give the same numbers up to rounding, with and without the silu epilogue."""
