@@ -183,6 +183,64 @@ def test_first_tokens_of_a_sequence(folders, dtype, tiny):
         check_logits(dtype, np.concatenate(got), want, what=rid)
 
 
+def _drawn_config(seed: int) -> dict:
+    """A configuration drawn from everything config.json allows: any group ratio, head sizes in
+    steps of 16 and a few that are only even, widths that are no multiple of 8, 16 or 64, tied or
+    untied heads, feed-forward widths whose 512-column phases share out unevenly."""
+    rng = np.random.default_rng(seed)
+    nkv = int(rng.choice([1, 2, 3, 4]))
+    nq = nkv * int(rng.choice([1, 2, 3, 4, 8]))
+    d = int(rng.choice([16, 32, 48, 64, 80, 96, 128, 144, 256, 24, 40]))
+    hidden = int(rng.choice([8, 24, 40, 64, 100, 136, 256, 520, 1024]))
+    inter = int(rng.choice([16, 56, 72, 256, 1000, 1536, 3072, 6152]))
+    return dict(
+        name=f"drawn{seed}", seed=seed, std=0.08, norm_std=0.1, page_size=int(rng.choice([8, 16, 32, 64])),
+        config=dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=int(rng.choice([1, 2])), hidden_size=hidden,
+                    num_attention_heads=nq, num_key_value_heads=nkv, head_dim=d, intermediate_size=inter,
+                    vocab_size=int(rng.choice([50, 257, 1000, 4099])), rope_theta=float(rng.choice([1e4, 1e6])),
+                    rms_norm_eps=float(rng.choice([1e-6, 1e-5])), tie_word_embeddings=bool(rng.integers(2)),
+                    max_position_embeddings=4096))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(20))
+def test_drawn_configurations(tmp_path, dtype, seed):
+    """Twenty drawn configurations: a prompt whole, one in two portions beside it, then both decoded
+    with 18 further requests of one token beside them (so the step has 20 rows: the matrix products
+    for 17..64 rows), everything against the plain implementation.  No size may be refused."""
+    tiny = _drawn_config(seed)
+    folder = make_folder(tiny, tmp_path)
+    cfg, w = plain_of(folder)
+    rng = np.random.default_rng(100 + seed)
+    ps = tiny["page_size"]
+    a = rng.integers(0, cfg["vocab_size"], size=41).tolist()
+    b = rng.integers(0, cfg["vocab_size"], size=37).tolist()
+    want_a, want_b = P.forward(w, cfg, a).numpy(), P.forward(w, cfg, b).numpy()
+    core = make_core(folder, dtype, ps, pages=20 * (-(-64 // ps)) + 4, seqs=20)
+    scale = max(float(np.abs(want_a).max()), float(np.abs(want_b).max()))
+    core.start_request("a")
+    core.start_request("b")
+    got = core.run([entry("a", a[:30]), entry("b", b[:9])]).cpu().numpy()
+    check_logits(dtype, got[:30], want_a[:30], scale, "a whole")
+    check_logits(dtype, got[30:], want_b[:9], scale, "b first portion")
+    got = core.run([entry("b", b[9:33])]).cpu().numpy()
+    check_logits(dtype, got, want_b[9:33], scale, "b second portion")
+    others = [f"o{i}" for i in range(18)]
+    for r in others:
+        core.start_request(r)
+    fed_a, fed_b = 30, 33
+    for step in range(4):
+        entries = [entry("a", a[fed_a:fed_a + 1]), entry("b", b[fed_b:fed_b + 1])]
+        entries += [entry(r, [int(rng.integers(0, cfg["vocab_size"]))], []) for r in others]
+        got = core.run(entries).cpu().numpy()
+        check_logits(dtype, got[0], want_a[fed_a], scale, f"a decoded {step}")
+        check_logits(dtype, got[1], want_b[fed_b], scale, f"b decoded {step}")
+        fed_a, fed_b = fed_a + 1, fed_b + 1
+    for r in ["a", "b"] + others:
+        core.finish_request(r)
+    core.cache.check_invariants()
+
+
 def test_step_function_refuses_bad_input(folders):
     from jax_vllm_amd.cache import OutOfPages
 
