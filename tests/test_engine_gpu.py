@@ -185,14 +185,14 @@ def test_first_tokens_of_a_sequence(folders, dtype, tiny):
 
 def _drawn_config(seed: int) -> dict:
     """A configuration drawn from everything config.json allows: any group ratio, head sizes in
-    steps of 16 and a few that are only even, widths that are no multiple of 8, 16 or 64, tied or
+    steps of 16 and a few that are only even, widths that are no multiple of 4, 8, 16 or 64, tied or
     untied heads, feed-forward widths whose 512-column phases share out unevenly."""
     rng = np.random.default_rng(seed)
     nkv = int(rng.choice([1, 2, 3, 4]))
     nq = nkv * int(rng.choice([1, 2, 3, 4, 8]))
     d = int(rng.choice([16, 32, 48, 64, 80, 96, 128, 144, 256, 24, 40]))
-    hidden = int(rng.choice([8, 24, 40, 64, 100, 136, 256, 520, 1024]))
-    inter = int(rng.choice([16, 56, 72, 256, 1000, 1536, 3072, 6152]))
+    hidden = int(rng.choice([6, 8, 24, 40, 50, 64, 100, 136, 256, 520, 1024]))
+    inter = int(rng.choice([16, 18, 50, 56, 72, 256, 1000, 1536, 3072, 6152]))
     return dict(
         name=f"drawn{seed}", seed=seed, std=0.08, norm_std=0.1, page_size=int(rng.choice([8, 16, 32, 64])),
         config=dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=int(rng.choice([1, 2])), hidden_size=hidden,
