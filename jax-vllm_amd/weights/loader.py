@@ -22,6 +22,13 @@ from .safetensors_io import open_shards
 TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 
 
+def torch_dtype(name: str) -> torch.dtype:
+    """The torch type of a dtype name in any spelling the engine configuration takes (bf16, fp32, ...)."""
+    from ..config.engine import canonical_dtype
+
+    return TORCH_DTYPES[canonical_dtype(name)]
+
+
 class WeightsError(ValueError):
     """The checkpoint does not fit the model: lists missing and unexpected tensors and wrong shapes."""
 
@@ -74,7 +81,7 @@ def load_model(folder, dtype: str = "bfloat16", device="cuda") -> tuple:
     arch, cfg, _ = resolve(folder)
     model = DecoderModel(arch.build_spec(cfg))
     specs, ignored = model.tensor_specs(), model.ignored_tensor_names()
-    compute = TORCH_DTYPES[dtype]
+    compute = torch_dtype(dtype)
     shards = list(open_shards(folder))
     owner, available = {}, {}
     for shard in shards:  # a later shard wins

@@ -17,7 +17,7 @@ import torch
 
 from ..config.registry import resolve
 from ..parts.model import DecoderModel
-from .loader import TORCH_DTYPES, target_dtype
+from .loader import target_dtype, torch_dtype
 from .safetensors_io import write_safetensors
 
 
@@ -46,7 +46,7 @@ def write_random_model(folder, config: Mapping, seed: int, std: float = 0.02, no
     folder.mkdir(parents=True, exist_ok=True)
     arch, cfg, raw = resolve(config)
     model = DecoderModel(arch.build_spec(cfg))
-    store = TORCH_DTYPES[dtype]
+    store = torch_dtype(dtype)
     records = []
     for name, ts in sorted(model.tensor_specs().items()):
         dt = torch.int32 if ts.role == "table" else store
@@ -68,7 +68,7 @@ def random_model_on_device(config: Mapping, seed: int, dtype: str = "bfloat16", 
         raw["num_hidden_layers"] = int(num_layers)
     arch, cfg, _ = resolve(raw)
     model = DecoderModel(arch.build_spec(cfg))
-    compute = TORCH_DTYPES[dtype]
+    compute = torch_dtype(dtype)
     tensors = {}
     for name, ts in model.tensor_specs().items():
         t = _draw(ts, seed, name, std, norm_std, device=device)
