@@ -3,8 +3,8 @@
 The reference's only command line is its HTTP server (``jllm/server.py:245-269``); the engine
 options here keep its names, defaults and meanings: ``--model-path`` (env ``JLLM_MODEL_PATH``),
 ``--max-num-seqs 4``, ``--max-model-len 2048``, ``--max-prefill-len 512``,
-``--dtype {bf16,fp32}``.  Server options (host, port, model name, prewarm) have no
-counterpart: there is no server and nothing to prewarm.  Added: the page geometry
+``--dtype {bf16,fp32}``, ``--no-prewarm``.  Server options (host, port, model name) have no
+counterpart: there is no server.  Added: the page geometry
 (``--block-size``, ``--num-blocks``, the arguments of the reference's ``make_driver``), the
 token budget of a step, sampling, and a random-weights mode.
 
@@ -33,6 +33,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--max-chunk", type=int, default=None, help="largest prompt portion of one request per step")
     p.add_argument("--no-prefix-cache", dest="prefix_cache", action="store_false")
     p.add_argument("--no-hip-graphs", dest="hip_graphs", action="store_false")
+    p.add_argument("--no-prewarm", dest="prewarm", action="store_false",
+                   help="Skip building the kernels and capturing the decode steps before the first prompt.")
     p.add_argument("--prompt-ids", action="append", default=[], metavar="'ID ID ...'",
                    help="one prompt as space- or comma-separated token ids (repeatable)")
     p.add_argument("--prompt-file", help="file with one prompt per line (token ids), or a JSON list of lists")
@@ -90,6 +92,8 @@ def main(argv=None) -> int:
               max_prefill_len=min(args.max_prefill_len, args.max_model_len),
               max_num_batched_tokens=args.max_num_batched_tokens, max_chunk=args.max_chunk,
               enable_prefix_cache=args.prefix_cache, use_hip_graphs=args.hip_graphs, seed=args.seed)
+    if args.prewarm:
+        print(f"prewarmed in {llm.prewarm():.2f}s", file=sys.stderr, flush=True)
     sp = SamplingParams(max_new_tokens=args.max_new_tokens, eos_id=args.eos_id, temperature=args.temperature)
     for out in llm.generate(prompts, sp):
         print(" ".join(str(t) for t in out), flush=True)

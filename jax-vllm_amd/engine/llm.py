@@ -147,6 +147,41 @@ class LLM(Engine):
         self.stats.graph_replays = self.core.graph_replays
         return events
 
+    def prewarm(self) -> float:
+        """Do now what the first requests would otherwise wait for, and return the seconds it took
+        (``jllm/engine/engine.py:182-208`` compiles its step programs for every batch shape there):
+        the kernel libraries this model needs are built or loaded, the library's matrix products
+        are initialised by one prompt portion, and the decode step is captured for every batch
+        bucket up to ``max_num_seqs`` at the smallest block-table width.  Only with no request
+        waiting or running; request ids, statistics and the prefix index are as before afterwards."""
+        import time
+
+        import torch
+
+        if self.has_work():
+            raise RuntimeError("prewarm needs an engine without waiting or running requests")
+        t0 = time.perf_counter()
+        from .core import _batch_bucket
+
+        saved = (self.stats, self._next_id, self.core.cache.prefix_cache)
+        self.core.cache.prefix_cache = False     # the warm-up prompts must not enter the prefix index
+        self.stats = self.scheduler.stats = EngineStats()
+        try:
+            buckets = sorted({_batch_bucket(n) for n in range(1, self.config.max_num_seqs + 1)
+                              if _batch_bucket(n) <= self.config.max_num_seqs} | {self.config.max_num_seqs})
+            room = min(self.config.prompt_limit, self.config.max_model_len - 4, self.config.max_num_batched_tokens)
+            first = True
+            for b in buckets:
+                n = max(1, min(room, 64)) if first else 1     # one real portion for the matrix library, then single tokens
+                first = False
+                self.generate([[0] * n] + [[0]] * (b - 1), SamplingParams(max_new_tokens=4))
+        finally:
+            self.core.cache.prefix_cache = saved[2]
+            self.stats, self._next_id = saved[0], saved[1]
+            self.scheduler.stats = self.stats
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
 
 # ---- the reference's functional spelling ------------------------------------------------
 def make_driver(model, max_num_seqs: int, max_model_len: int, max_prefill_len: Optional[int] = None,
@@ -167,3 +202,8 @@ def has_work(driver: LLM) -> bool:
 
 def step(driver: LLM) -> list:
     return driver.step()
+
+
+def prewarm(driver: LLM) -> float:
+    """``jllm/engine/engine.py:182-208``: seconds spent on what the first requests would wait for."""
+    return driver.prewarm()

@@ -55,6 +55,43 @@ def test_greedy_generation_workload_a(folders, dtype):
     assert out == got[1]
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prewarm_leaves_the_engine_as_it_was(folders, dtype):
+    """``prewarm`` (the reference's ``jllm/engine/engine.py:182-208``) captures the decode step for
+    every batch bucket and then leaves no trace: request ids start at 0, the counters are zero,
+    nothing is in the prefix index, all pages are free, and generation gives the same tokens as
+    an engine that was not warmed."""
+    from jax_vllm_amd import LLM, SamplingParams, prewarm
+
+    cfg, w = plain_of(folders["B"])
+    rng = np.random.default_rng(9)
+    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (3, 20, 41)]
+    opts = dict(dtype=dtype, block_size=TINY_B["page_size"], max_num_seqs=5, max_model_len=96, max_num_batched_tokens=64)
+    cold = LLM(folders["B"], **opts)
+    warm = LLM(folders["B"], **opts)
+    pool = warm.core.cache.groups[0].pool
+    free = pool.num_free
+    seconds = prewarm(warm)
+    assert seconds > 0 and not warm.has_work() and warm.requests == {}
+    assert warm.stats.steps_run == 0 and warm.stats.emitted_tokens == 0 and warm.stats.admissions == 0
+    assert len(warm.core._graphs) >= 3                       # buckets 1, 2, 4 (and 5 rows in the bucket of 8)
+    warm.core.cache.check_invariants()
+    assert pool.num_free == free and not pool._by_hash       # all pages free, none indexed by content
+    assert warm.add_request(prompts[0], SamplingParams(max_new_tokens=2)) == 0
+    warm.abort_all()
+    sp = SamplingParams(max_new_tokens=12)
+    got_warm, got_cold = warm.generate(prompts, sp), cold.generate(prompts, sp)
+    assert warm.stats.cache_hit_tokens == 0
+    if dtype == "float32":
+        assert got_warm == got_cold
+    for p, g in zip(prompts, got_warm):
+        check_tokens_follow(dtype, cfg, w, p, g)
+    with pytest.raises(RuntimeError):
+        warm.add_request(prompts[1], sp)
+        warm.prewarm()
+    warm.abort_all()
+
+
 def test_temperature_generation_workload_b_is_cut_independent(folders):
     """BASELINE workload B: prompts 1/9/40/64/100 (two share a 32-token prefix), arrivals at steps
     0,0,2,3,5, budget 24, temperature 0.8, seed 7, 20 new tokens.  The draws are keyed by
