@@ -3,12 +3,13 @@ from .config import ConfigError, EngineConfig, Qwen3Config
 from .engine.request import EngineStats, Request, SamplingParams, StepEvent
 
 __all__ = ["ConfigError", "EngineConfig", "Qwen3Config", "EngineStats", "Request", "SamplingParams", "StepEvent",
-           "LLM", "make_driver", "add_request", "has_work", "step", "prewarm", "load_model", "write_random_model"]
+           "LLM", "make_driver", "add_request", "has_work", "step", "prewarm", "start", "stop", "stream",
+           "load_model", "write_random_model"]
 
 
 def __getattr__(name):
     # the engine and the weight loader pull in torch and the kernels: loaded on first use
-    if name in ("LLM", "make_driver", "add_request", "has_work", "step", "prewarm"):
+    if name in ("LLM", "make_driver", "add_request", "has_work", "step", "prewarm", "start", "stop", "stream"):
         from .engine import llm
 
         return getattr(llm, name)

@@ -92,6 +92,29 @@ def test_prewarm_leaves_the_engine_as_it_was(folders, dtype):
     warm.abort_all()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_streaming_from_a_background_loop(folders, dtype):
+    """The engine stepped in a thread of its own (``start`` / ``stream`` / ``stop``) gives the tokens
+    of the blocking loop, captured decode steps included."""
+    from jax_vllm_amd import LLM, SamplingParams, start, stop, stream
+
+    cfg, w = plain_of(folders["A"])
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (4, 19, 33)]
+    llm = LLM(folders["A"], dtype=dtype, block_size=TINY_A["page_size"], max_num_seqs=3, max_model_len=64,
+              max_num_batched_tokens=32)
+    sp = SamplingParams(max_new_tokens=10)
+    want = llm.generate(prompts, sp)
+    start(llm)
+    rids = [llm.add_request(p, sp) for p in prompts]
+    got = [[ev.token for ev in stream(llm, r)] for r in rids]
+    stop(llm)
+    assert got == want
+    for p, g in zip(prompts, got):
+        check_tokens_follow(dtype, cfg, w, p, g)
+    assert llm.generate(prompts[:1], sp) == want[:1]          # and the blocking loop works again afterwards
+
+
 def test_temperature_generation_workload_b_is_cut_independent(folders):
     """BASELINE workload B: prompts 1/9/40/64/100 (two share a 32-token prefix), arrivals at steps
     0,0,2,3,5, budget 24, temperature 0.8, seed 7, 20 new tokens.  The draws are keyed by

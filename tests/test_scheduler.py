@@ -272,3 +272,45 @@ def test_random_workloads_with_few_pages_finish_right(seed):
     assert got == [expected(p, k) for p, k in zip(prompts, new)]
     core.cache.check_invariants()
     assert core.cache.num_free_pages() == eng.config.usable_pages
+
+
+def test_background_loop_streams_what_the_blocking_loop_generates():
+    """``start`` / ``stream`` / ``stop`` (the reference's threaded use, jllm/engine/engine.py:134-233):
+    requests added while the loop runs in its own thread give the same tokens as ``generate``,
+    every stream ends with the finishing event, and the thread sleeps without work."""
+    prompts = [[1, 2, 3], list(range(40)), [7] * 17]
+    sp = SamplingParams(max_new_tokens=9)
+    blocking, _ = make(max_num_seqs=2, max_model_len=128, block_size=8, max_num_batched_tokens=16)
+    want = blocking.generate(prompts, sp)
+    eng, _ = make(max_num_seqs=2, max_model_len=128, block_size=8, max_num_batched_tokens=16)
+    eng.start()
+    eng.start()                                   # a second start changes nothing
+    rids = [eng.add_request(p, sp) for p in prompts]
+    got = []
+    for rid in reversed(rids):                    # drained in another order than they were added
+        events = list(eng.stream(rid))
+        assert [e.request_id for e in events] == [rid] * 9 and [e.finished for e in events] == [False] * 8 + [True]
+        got.append([e.token for e in events])
+    assert got[::-1] == want and not eng.has_work() and eng.requests == {}
+    with pytest.raises(KeyError):
+        next(eng.stream(rids[0]))                 # already drained
+    late = eng.add_request([5, 6], SamplingParams(max_new_tokens=3))     # the sleeping thread wakes up
+    assert len(list(eng.stream(late))) == 3
+    eng.stop()
+    assert eng._thread is None
+
+
+def test_background_loop_hands_its_failure_to_the_caller():
+    eng, core = make(max_num_seqs=2, max_model_len=64, block_size=8, max_num_batched_tokens=16)
+
+    def broken(entries, borrow=False):
+        raise ValueError("the step function broke")
+
+    eng._run = broken
+    eng.start()
+    rid = eng.add_request([1, 2, 3], SamplingParams(max_new_tokens=4))
+    with pytest.raises(RuntimeError, match="the step function broke"):
+        list(eng.stream(rid))
+    with pytest.raises(RuntimeError, match="engine loop failed"):
+        eng.add_request([4], SamplingParams(max_new_tokens=1))
+    eng.stop()
