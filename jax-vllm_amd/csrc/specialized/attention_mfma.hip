@@ -88,6 +88,7 @@ struct AttnArgs {
 // barriers.  Keys are masked only on tiles that cross a row's causal limit or window edge.
 constexpr int RT = D <= 128 ? 2 : 1;       // row groups per block = row tiles per wave
 constexpr int GROUP_ROWS = 64;             // 4 waves x 16 rows
+constexpr float RESCALE_STEP = 8.f;        // growth of a row's maximum (powers of two) that moves its reference: p <= 2^8
 constexpr int KCH = BN * (DK / 8);         // 16-byte pieces of a K tile
 constexpr int VCH = D * (BN / 8);          // 16-byte pieces of a V^T tile
 constexpr int KPT = (KCH + 255) / 256;     // pieces per thread
@@ -198,11 +199,12 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
   load_table(j_first);
   __syncthreads();
 
-  float m_run[RT], l_lane[RT];
+  float m_run[RT], m_ref[RT], l_lane[RT];
   f32x4 acc[RT][NDT];
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     m_run[t] = -INFINITY;
+    m_ref[t] = -INFINITY;
     l_lane[t] = 0.f;
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt) acc[t][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -401,8 +403,20 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
       tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
       const float m_new = fmaxf(m_run[t], tmax);                       // raw-score units
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
-      const float alpha = fast_exp2(m_run[t] * p.scale_log2 - m_use);  // exp2(-inf) = 0 on the first tile
+      m_run[t] = m_new;
+      // The exponents are taken against m_ref, which follows the running maximum only when that
+      // has grown by more than RESCALE_STEP (in powers of two): sums and outputs are then brought
+      // to the new reference.  Most tiles change no row's reference and skip that work; a row's
+      // numbers do not depend on the other rows of its wave, only the skipping does.
+      const bool grown = (m_new - m_ref[t]) * p.scale_log2 > RESCALE_STEP;   // false while no key is visible
+      if (__builtin_amdgcn_ballot_w64(grown) != 0) {
+        const float alpha = grown ? fast_exp2((m_ref[t] - m_new) * p.scale_log2) : 1.f;   // 0 from -inf
+        if (grown) m_ref[t] = m_new;
+        l_lane[t] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) acc[t][dt] *= alpha;
+      }
+      const float m_use = (m_ref[t] == -INFINITY) ? 0.f : m_ref[t] * p.scale_log2;
       float psum = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
@@ -412,10 +426,7 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
           s[t][kt][e] = pv;
           psum += pv;
         }
-      l_lane[t] = l_lane[t] * alpha + psum;
-      m_run[t] = m_new;
-#pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) acc[t][dt] *= alpha;
+      l_lane[t] += psum;
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk)
 #pragma unroll

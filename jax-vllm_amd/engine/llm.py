@@ -230,10 +230,11 @@ class LLM(Engine):
         self.core = EngineCore(self.model, config)
         self.sampler = Sampler(self.core.device)
         super().__init__(config, self.core.cache, self.core.run, self.sampler.sample, self.core.vocab_size)
+        self._replays_before = 0     # replays of a prewarm are not the requests'
 
     def step(self) -> list:
         events = super().step()
-        self.stats.graph_replays = self.core.graph_replays
+        self.stats.graph_replays = self.core.graph_replays - self._replays_before
         return events
 
     def prewarm(self) -> float:
@@ -268,6 +269,7 @@ class LLM(Engine):
             self.core.cache.prefix_cache = saved[2]
             self.stats, self._next_id = saved[0], saved[1]
             self.scheduler.stats = self.stats
+            self._replays_before = self.core.graph_replays
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 

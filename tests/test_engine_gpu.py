@@ -74,6 +74,7 @@ def test_prewarm_leaves_the_engine_as_it_was(folders, dtype):
     seconds = prewarm(warm)
     assert seconds > 0 and not warm.has_work() and warm.requests == {}
     assert warm.stats.steps_run == 0 and warm.stats.emitted_tokens == 0 and warm.stats.admissions == 0
+    assert warm.stats.graph_replays == 0
     assert len(warm.core._graphs) >= 3                       # buckets 1, 2, 4 (and 5 rows in the bucket of 8)
     warm.core.cache.check_invariants()
     assert pool.num_free == free and not pool._by_hash       # all pages free, none indexed by content
