@@ -1,5 +1,6 @@
-"""The layer sizes of a real model (Qwen3-8B: hidden 4096, 32/8 heads of 128, feed-forward
-12288, vocabulary 151936) with two layers of random weights: the 32-bit path and the bfloat16
+"""The layer sizes of real models (Qwen3-8B: hidden 4096, 32/8 heads of 128, feed-forward
+12288, vocabulary 151936; and the 14B sizes: hidden 5120, 40/8 heads, feed-forward 17408) with two
+layers of random weights: the 32-bit path and the bfloat16
 path against the plain implementation, whole, token by token, in portions and mixed.  These are
 the sizes at which the kernels' wide paths run (16-byte norm loads, the streaming matrix
 product's real shapes, a vocabulary that is no power of two, the 128-wide MFMA attention)."""
@@ -15,10 +16,14 @@ pytestmark = pytest.mark.gpu
 CONFIG = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=2, hidden_size=4096, num_attention_heads=32,
               num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
               rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960)
+# the next size up: 5 query heads per kv head, a width of 5120 (inner sizes that are no multiple of
+# 4096: other organisations of the streaming products), a feed-forward of 17408
+CONFIG_14B = dict(CONFIG, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
 
 
-@pytest.fixture(scope="module")
-def big():
+@pytest.fixture(scope="module", params=[CONFIG, CONFIG_14B], ids=["8b", "14b"])
+def big(request):
+    CONFIG = request.param
     from jax_vllm_amd.config import resolve
     from jax_vllm_amd.parts import DecoderModel
     from jax_vllm_amd.weights.random_init import _draw
