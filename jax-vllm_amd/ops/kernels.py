@@ -374,7 +374,7 @@ def gemm_tile64(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
 _cu_count = {}
 
 
-def _compute_units(device) -> int:
+def compute_units(device) -> int:
     n = _cu_count.get(device)
     if n is None:
         n = _cu_count[device] = torch.cuda.get_device_properties(device).multi_processor_count
@@ -431,7 +431,7 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     """
     if k % 8:
         return None
-    cus = _compute_units(device) if device is not None else 256
+    cus = compute_units(device) if device is not None else 256
     narrow = partial_ok and not silu_pairs and n % 4 == 0 and n <= PARTIAL_SUM_MAX_WIDTH
     if m > SKINNY_AUTO_ROWS:
         if narrow and m <= SKINNY_MAX_ROWS:

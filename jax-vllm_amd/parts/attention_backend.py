@@ -79,15 +79,27 @@ def prefill_work_items(q_lens, context_lens, g: int, window: int, group_rows: in
     return [(r, a, b) for _, r, a, b in items]
 
 
+def prefill_item_shape(rows: int, nkv: int, group_rows: int, kernel_groups: int, compute_units: int):
+    """(groups per work item, whether light groups are paired with heavy ones) for a step with
+    ``rows`` (query, head-in-group) rows per kv head in its prompt portions.  Measured on 32 q heads,
+    8 kv heads of 128: while items of two groups would not even give every compute unit a block,
+    items of one group do better although every block then loads its keys for half the rows
+    (512 tokens after 3,000: 111 against 135 us; after 16,000: 507 against 622); balancing wins
+    while the blocks fit on the chip about one and a half times (2,048 tokens: 87 against 102 us),
+    sharing keys between neighbours wins beyond (8,192: 887 against 1,036)."""
+    blocks = -(-rows // (group_rows * kernel_groups)) * nkv
+    if kernel_groups > 1 and blocks <= compute_units:
+        return 1, True
+    return kernel_groups, blocks <= BALANCE_BLOCKS
+
+
 def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> MfmaPlan:
     g = nq // nkv
-    group_rows, groups_per_item = K.attn_prefill_geometry(head_dim)
-    # measured on 32 q heads, 8 kv heads of 128: balancing wins while the blocks fit on the chip about
-    # one and a half times (2,048 tokens: 87 against 102 us), sharing wins beyond (8,192: 887 against 1,036)
+    group_rows, kernel_groups = K.attn_prefill_geometry(head_dim)
     rows = sum(ql * g for ql in ctx.q_lens_host if ql > 1)
-    blocks = -(-rows // (group_rows * groups_per_item)) * nkv
+    groups_per_item, balance = prefill_item_shape(rows, nkv, group_rows, kernel_groups, K.compute_units(device))
     prefill = prefill_work_items(ctx.q_lens_host, ctx.context_lens_host, g, window, group_rows, groups_per_item,
-                                 balance=blocks <= BALANCE_BLOCKS)
+                                 balance=balance)
     decode = [r for r, ql in enumerate(ctx.q_lens_host) if ql == 1]
     max_kv_decode = max([ctx.context_lens_host[r] + 1 for r in decode], default=1)
     splits = decode_splits(len(decode), nkv * (-(-g // 16)), max_kv_decode) if decode else 1

@@ -1,7 +1,8 @@
 """The host-side plan of the prefill attention kernel: which rows go to which block."""
 import random
 
-from jax_vllm_amd.parts.attention_backend import KEY_TILE, decode_splits, prefill_work_items
+from jax_vllm_amd.parts.attention_backend import (BALANCE_BLOCKS, KEY_TILE, decode_splits, prefill_item_shape,
+                                                   prefill_work_items)
 
 
 def _tiles(cl, m0, ql, g, rows, window):
@@ -52,3 +53,17 @@ def test_decode_splits_fill_the_chip_but_keep_a_tile_per_wave():
     assert decode_splits(1, 8, 100) == 1                     # too few keys to share out
     assert decode_splits(1, 8, 8192) == 64
     assert decode_splits(64, 8, 8192) == 1                   # enough blocks already
+
+
+def test_item_shape_follows_the_fill_of_the_chip():
+    """Few rows: items of one group, so that more blocks than compute units exist at all; more:
+    two groups, light paired with heavy; many: two neighbouring groups."""
+    shape = lambda tokens: prefill_item_shape(tokens * 4, 8, 64, 2, 256)     # 32 q heads over 8 kv heads
+    assert shape(512) == (1, True) and shape(1024) == (1, True)          # 128 and 256 blocks of two groups
+    assert shape(2048) == (2, True)                                      # 512 blocks
+    assert shape(8192) == (2, False) and 8192 * 4 // 128 * 8 > BALANCE_BLOCKS
+    assert prefill_item_shape(100, 8, 64, 1, 256) == (1, True)           # a kernel with one group per item stays so
+    # every row still lands in exactly one item
+    items = prefill_work_items([600], [37], 4, 0, 64, 1)
+    rows = sorted(m0 for _, m0, other in items if other == -1)
+    assert rows == list(range(0, 600 * 4, 64)) and all(other == -1 for _, _, other in items)
