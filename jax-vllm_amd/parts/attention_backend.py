@@ -20,7 +20,7 @@ from ..ops import kernels as K
 
 TARGET_BLOCKS = 512          # about two blocks per compute unit
 MIN_KEYS_PER_SPLIT = 128     # one 32-key tile for each of a block's 4 waves
-BALANCE_BLOCKS = 768         # up to here prefill work items pair light row groups with heavy ones
+RESIDENT_BLOCKS = 2          # blocks of the prefill kernel that a compute unit holds at once
 
 
 @dataclass
@@ -85,12 +85,14 @@ def prefill_item_shape(rows: int, nkv: int, group_rows: int, kernel_groups: int,
     8 kv heads of 128: while items of two groups would not even give every compute unit a block,
     items of one group do better although every block then loads its keys for half the rows
     (512 tokens after 3,000: 111 against 135 us; after 16,000: 507 against 622); balancing wins
-    while the blocks fit on the chip about one and a half times (2,048 tokens: 87 against 102 us),
-    sharing keys between neighbours wins beyond (8,192: 887 against 1,036)."""
+    while all blocks are on the chip at once, two per compute unit (2,048 tokens, 512 blocks: 88
+    against 98 us); one more block and the equal loads need a whole further round, so neighbours
+    that share their keys, heaviest first, win from there (2,304 tokens, 576 blocks: 111 against
+    137 us; 8,192: 887 against 1,036)."""
     blocks = -(-rows // (group_rows * kernel_groups)) * nkv
     if kernel_groups > 1 and blocks <= compute_units:
         return 1, True
-    return kernel_groups, blocks <= BALANCE_BLOCKS
+    return kernel_groups, blocks <= RESIDENT_BLOCKS * compute_units
 
 
 def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> MfmaPlan:

@@ -1,8 +1,7 @@
 """The host-side plan of the prefill attention kernel: which rows go to which block."""
 import random
 
-from jax_vllm_amd.parts.attention_backend import (BALANCE_BLOCKS, KEY_TILE, decode_splits, prefill_item_shape,
-                                                   prefill_work_items)
+from jax_vllm_amd.parts.attention_backend import KEY_TILE, decode_splits, prefill_item_shape, prefill_work_items
 
 
 def _tiles(cl, m0, ql, g, rows, window):
@@ -60,8 +59,8 @@ def test_item_shape_follows_the_fill_of_the_chip():
     two groups, light paired with heavy; many: two neighbouring groups."""
     shape = lambda tokens: prefill_item_shape(tokens * 4, 8, 64, 2, 256)     # 32 q heads over 8 kv heads
     assert shape(512) == (1, True) and shape(1024) == (1, True)          # 128 and 256 blocks of two groups
-    assert shape(2048) == (2, True)                                      # 512 blocks
-    assert shape(8192) == (2, False) and 8192 * 4 // 128 * 8 > BALANCE_BLOCKS
+    assert shape(2048) == (2, True)                                      # 512 blocks: all on the chip at once
+    assert shape(2304) == (2, False) and shape(8192) == (2, False)       # one more round of blocks
     assert prefill_item_shape(100, 8, 64, 1, 256) == (1, True)           # a kernel with one group per item stays so
     # every row still lands in exactly one item
     items = prefill_work_items([600], [37], 4, 0, 64, 1)
