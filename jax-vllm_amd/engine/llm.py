@@ -199,8 +199,10 @@ class Engine:
         while self.has_work():
             self.step()
         outs = [list(self.requests[r].output_ids) for r in rids]
-        for r in rids:
-            del self.requests[r]
+        with self._wake:
+            for r in rids:
+                del self.requests[r]
+                self._streams.pop(r, None)     # made if the background loop is running too
         return outs
 
 
