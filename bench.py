@@ -3,7 +3,7 @@ prefill tokens/s at 2,048 tokens and decode at batch 1 and 64 beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--shape 8b|14b|32b]
 
-The model has the layer sizes of BASELINE.json ``configs[2]`` (Qwen3-8B shape) with random
+The model has the layer sizes of Qwen3-8B (the headline configuration) with random
 weights drawn on the device; prompts are seeded uniform-random token ids of 1,024 tokens;
 a "step" is one decode step of the whole engine (scheduler, step function, sampling).
 It prints ONE JSON line.  More than one GPU is not supported: it says so and exits with 2.
@@ -29,7 +29,7 @@ QWEN3_8B = dict(
     num_key_value_heads=8, head_dim=128, intermediate_size=12288, vocab_size=151936, rope_theta=1000000.0,
     rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=40960,
 )
-# the other shapes of BASELINE.json (configs[3] and [4]), for runs at further sizes: --shape
+# the layer sizes of Qwen3-14B and Qwen3-32B, for runs at further sizes: --shape
 SHAPES = {
     "8b": ("Qwen3-8B-shaped", QWEN3_8B),
     "14b": ("Qwen3-14B-shaped", dict(QWEN3_8B, num_hidden_layers=40, hidden_size=5120, num_attention_heads=40,
@@ -101,7 +101,7 @@ def measure_prefill(llm, rng, vocab, repeats=3):
 
 
 def measure_mixed(llm, rng, vocab, running=32, joining=4, join_len=3000, shared=1024):
-    """The continuous-batching mix of BASELINE.json configs[3]: ``running`` requests decode at contexts
+    """A continuous-batching mix: ``running`` requests decode at contexts
     uniform in [512, 4096] when ``joining`` prompts of ``join_len`` tokens arrive, two of which share
     their first ``shared`` tokens; timed from their arrival until all of them have their first token."""
     from jax_vllm_amd import SamplingParams

@@ -30,7 +30,7 @@ def entry(rid, tokens, want=None):
 # ------------------------------------------------------------------ generation through the entry point
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_greedy_generation_workload_a(folders, dtype):
-    """BASELINE workload A: 3 requests, prompts of 5, 17 and 33 random ids, greedy, 16 new tokens."""
+    """Workload A: 3 requests, prompts of 5, 17 and 33 random ids, greedy, 16 new tokens."""
     from jax_vllm_amd import LLM, SamplingParams
 
     cfg, w = plain_of(folders["A"])
@@ -117,7 +117,7 @@ def test_streaming_from_a_background_loop(folders, dtype):
 
 
 def test_temperature_generation_workload_b_is_cut_independent(folders):
-    """BASELINE workload B: prompts 1/9/40/64/100 (two share a 32-token prefix), arrivals at steps
+    """Workload B: prompts 1/9/40/64/100 (two share a 32-token prefix), arrivals at steps
     0,0,2,3,5, budget 24, temperature 0.8, seed 7, 20 new tokens.  The draws are keyed by
     (seed, request, index), so another budget, batch width or page pool gives the same tokens."""
     from jax_vllm_amd import LLM, SamplingParams
