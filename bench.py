@@ -153,8 +153,9 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
                     help="with --only decode: prompt length of the decoding requests (long-context runs)")
     args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {max(args.gpus, world)} is not supported")
         sys.exit(2)
 
     import numpy as np
