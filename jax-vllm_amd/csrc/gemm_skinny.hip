@@ -331,31 +331,33 @@ static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, i
 }
 
 // ---------------------------------------------------------------------------------------------
-// Third organisation, for at most 16 rows of x and an inner size of at most 8 * NL * 32: blocks
-// that stay.  Each of a block's 8 waves keeps ITS slice of x (NL steps of 32 columns) in registers
+// Third organisation, for at most 16 rows of x (32 with NL <= 8: two row tiles) and an inner size
+// of at most 8 * NL * 32: blocks that stay.  Each of a block's 8 waves keeps ITS slice of x (NL steps of 32 columns) in registers
 // as MFMA B operands for the whole kernel, so the loop over the block's row tiles of W touches
 // LDS only to add the 8 waves' partial tiles: no staging of x, no barrier between the loads.
 // The next tile's weights are asked for before the current tile is multiplied and reduced.
 // A longer inner size is shared out to gridDim.y groups of blocks, 8 * NL * 32 columns each,
 // which write float partial products to y + group * M * ldy (added by the reader, in order).
-template <int NL, typename OutT, bool PAIRS>
+template <int NL, int MT, typename OutT, bool PAIRS>
 __global__ void __launch_bounds__(512)
 gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
                               int M, int N, int K, long long ldx, long long ldy) {
   y += (long long)blockIdx.y * M * ldy;
-  __shared__ __attribute__((aligned(16))) float red[8 * 256];
+  __shared__ __attribute__((aligned(16))) float red[8 * MT * 256];
   const int tid = threadIdx.x;
   const int wk = tid >> 6, lane = tid & 63, li = lane & 15, lc = lane >> 4;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   const int k0 = (blockIdx.y * 8 + wk) * NL * 32 + lc * 8;     // this lane's first column
   const int n_tiles = (N + 15) / 16;
-  // x: row li (zero beyond M), this wave's columns
-  bf16x8 b[NL];
+  // x: rows mt * 16 + li (zero beyond M), this wave's columns
+  bf16x8 b[MT][NL];
 #pragma unroll
-  for (int i = 0; i < NL; ++i) {
-    const int k = k0 + i * 32;
-    b[i] = (li < M && k < K) ? *(const bf16x8*)(x + (long long)li * ldx + k) : zero;
-  }
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+      const int k = k0 + i * 32, m = mt * 16 + li;
+      b[mt][i] = (m < M && k < K) ? *(const bf16x8*)(x + (long long)m * ldx + k) : zero;
+    }
   auto load_tile = [&](int tile, bf16x8 (&a)[NL]) {
     const int n = tile * 16 + li;
     const bf16_t* wrow = W + (long long)(n < N ? n : 0) * K + k0;
@@ -363,29 +365,35 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
     for (int i = 0; i < NL; ++i) a[i] = (n < N && k0 + i * 32 < K) ? *(const bf16x8*)(wrow + i * 32) : zero;
   };
   auto finish_tile = [&](int tile, bf16x8 (&a)[NL]) {
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[MT];
 #pragma unroll
-    for (int i = 0; i < NL; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[i], acc, 0, 0, 0);
-    *(f32x4*)(red + (wk * 256 + lane * 4)) = acc;
+    for (int mt = 0; mt < MT; ++mt) {
+      acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < NL; ++i) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[mt][i], acc[mt], 0, 0, 0);
+      *(f32x4*)(red + ((wk * MT + mt) * 256 + lane * 4)) = acc[mt];
+    }
     __syncthreads();
-    if (wk == 0) {
-      f32x4 s = acc;                               // fixed order: wave 0, 1, ..., 7
+    if (wk < MT) {                                 // wave mt adds row tile mt, in fixed order: wave 0, 1, ..., 7
+      const int mt = wk;
+      f32x4 s = *(const f32x4*)(red + (mt * 256 + lane * 4));
 #pragma unroll
       for (int w = 1; w < 8; ++w) {
-        const f32x4 t = *(const f32x4*)(red + (w * 256 + lane * 4));
+        const f32x4 t = *(const f32x4*)(red + ((w * MT + mt) * 256 + lane * 4));
         s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
       }
-      const int nb = tile * 16 + lc * 4;           // the accumulator holds y^T[n = lc*4+e][m = li]
-      if (li < M) {
+      const int nb = tile * 16 + lc * 4;           // the accumulator holds y^T[n = lc*4+e][m = mt*16 + li]
+      const int m = mt * 16 + li;
+      if (m < M) {
         if (PAIRS) {
 #pragma unroll
           for (int e = 0; e < 4; e += 2)
             if (nb + e + 1 < N)
-              y[(long long)li * ldy + (nb + e) / 2] = from_f32<OutT>(s[e] / (1.f + expf(-s[e])) * s[e + 1]);
+              y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(s[e] / (1.f + expf(-s[e])) * s[e + 1]);
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (nb + e < N) y[(long long)li * ldy + nb + e] = from_f32<OutT>(s[e]);
+            if (nb + e < N) y[(long long)m * ldy + nb + e] = from_f32<OutT>(s[e]);
         }
       }
     }
@@ -407,33 +415,42 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
   }
 }
 
-template <int NL, typename OutT, bool PAIRS>
+template <int NL, int MT, typename OutT, bool PAIRS>
 static int launch_persistent(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
                              long long ldy, int blocks, int ksplit, hipStream_t stream) {
   const int n_tiles = (N + 15) / 16;
   blocks = (blocks + ksplit - 1) / ksplit;           // per group
   if (blocks > n_tiles) blocks = n_tiles;
-  hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, OutT, PAIRS>), dim3(blocks, ksplit), dim3(512), 0, stream,
-                     (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
+  hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS>), dim3(blocks, ksplit), dim3(512), 0,
+                     stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
   return JV_LAUNCH_CHECK();
 }
 
 // wr == -2: nks = NL in {4, 5, 8, 10, 12, 16, 17}, wk = blocks in all; the inner size must be at most
-// ksplit * 8 * NL * 32 and more than (ksplit - 1) * 8 * NL * 32
+// ksplit * 8 * NL * 32 and more than (ksplit - 1) * 8 * NL * 32.  Up to 16 rows with every NL, up
+// to 32 rows (two row tiles of x in registers) with NL <= 8.
 template <typename OutT, bool PAIRS>
 static int dispatch_persistent(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
                                long long ldy, int blocks, int ksplit, hipStream_t s) {
-  if (M > 16 || blocks < 1 || ksplit > 65535 || K > (long long)ksplit * 8 * nl * 32 ||
+  if (M > 32 || (M > 16 && nl > 8) || blocks < 1 || ksplit > 65535 || K > (long long)ksplit * 8 * nl * 32 ||
       K <= (long long)(ksplit - 1) * 8 * nl * 32)
     return (int)hipErrorInvalidValue;
+  if (M > 16) {
+    switch (nl) {
+      case 4: return launch_persistent<4, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+      case 5: return launch_persistent<5, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+      case 8: return launch_persistent<8, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    }
+    return (int)hipErrorInvalidValue;
+  }
   switch (nl) {
-    case 4: return launch_persistent<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 5: return launch_persistent<5, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 8: return launch_persistent<8, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 10: return launch_persistent<10, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 12: return launch_persistent<12, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 16: return launch_persistent<16, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 17: return launch_persistent<17, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 4: return launch_persistent<4, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 5: return launch_persistent<5, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 8: return launch_persistent<8, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 10: return launch_persistent<10, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 12: return launch_persistent<12, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 16: return launch_persistent<16, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 17: return launch_persistent<17, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
   }
   return (int)hipErrorInvalidValue;
 }

@@ -311,13 +311,15 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     _need(m <= SKINNY_MAX_ROWS, f"gemm_skinny takes at most {SKINNY_MAX_ROWS} rows")
     _need(k % 8 == 0, "the inner size must be a multiple of 8")
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
-    _need(block_shape[0] != -2 or (m <= 16 and block_shape[2] in STAY_PIECES
+    _need(block_shape[0] != -2 or ((m <= 16 or (m <= 32 and block_shape[2] <= 8)) and block_shape[2] in STAY_PIECES
                                    and 256 * block_shape[2] * (ksplit - 1) < k <= 256 * block_shape[2] * ksplit),
-          "the organisation with blocks that stay takes at most 16 rows and an inner size of ksplit * 256 * pieces at most")
+          "the organisation with blocks that stay takes at most 16 rows (32 with at most 8 pieces) and an inner "
+          "size of ksplit * 256 * pieces at most")
     _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
           "the silu epilogue writes bfloat16, needs an even number of rows of w and the chunked organisation")
-    _need(ksplit >= 1 and (ksplit == 1 or (block_shape[0] in (-1, -2) and out_dtype == torch.float32 and m <= 16)),
-          "sharing the inner size out needs the resident organisation, float32 output and at most 16 rows")
+    _need(ksplit >= 1 and (ksplit == 1 or (block_shape[0] in (-1, -2) and out_dtype == torch.float32
+                                           and (m <= 16 or block_shape[0] == -2))),
+          "sharing the inner size out needs x resident (at most 16 rows) or blocks that stay, and float32 output")
     n_out = n // 2 if silu_pairs else n
     shape = (m, n_out) if ksplit == 1 else (ksplit, m, n_out)
     if out is None:
@@ -423,6 +425,10 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     * the same at 17..64 rows when every block gets at least 3,072 columns: blocks of 64 rows of w,
       one per compute unit (the feed-forward's second product: 4,096 x 12,288 at 64 rows 30 us
       against the library's 37; 5,120 x 17,408 65 against 131; 5,120 x 25,600 91 against 157);
+    * 17..32 rows against narrow matrices with a short inner size (the attention's output product):
+      staying blocks with two row tiles of x in registers, the inner size shared out to 4 groups
+      (4,096 x 4,096 at 32 rows: 10.8 us against the library's 13.0; at 33..64 rows the four row
+      tiles pull x through the caches too often: the library's);
     * one or two rows against wide matrices: x resident in LDS (chosen inside the kernel library);
     * 9..16 rows of a large matrix that fits none of these: the library (its wider tiles amortise
       x), unless the inner size is beyond 12,288, where the library needs 113 us for the 178 MB
@@ -438,6 +444,9 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
             parts = _fit_parts(-(-k // 256), min(4, cus // -(-n // 64)))
             if parts >= 2 and k >= parts * TILE64_MIN_SHARE:
                 return TILE64, parts
+            nl = _stay_pieces(k, 4)
+            if m <= 32 and nl is not None and nl <= 8 and -(-n // 16) * 2 <= PARTIAL_BLOCKS:
+                return (-2, cus, nl), 4
         return None
     tiles = -(-n // 16)
     if narrow and tiles * 2 <= PARTIAL_BLOCKS:

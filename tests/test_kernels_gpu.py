@@ -676,7 +676,8 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     (8, 24576, 512, (0, 0, 0)), (48, 6144, 1024, (4, 2, 2)), (1, 6144, 4096, (1, 8, 4)), (9, 160, 4096, (4, 4, 8)),
     (1, 8200, 4096, (0, 0, 0)), (2, 100, 4096, (-1, 8, 16)), (8, 333, 1000, (-1, 16, 4)), (16, 64, 12288, (-1, 4, 8)),
     (11, 50, 72, (-1, 3, 4)), (8, 24576, 512, (-2, 64, 4)), (16, 333, 4096, (-2, 7, 16)), (5, 777, 2000, (-2, 1000, 8)),
-    (3, 100, 72, (-2, 3, 4)), (1, 8200, 4096, (-2, 256, 16))])
+    (3, 100, 72, (-2, 3, 4)), (1, 8200, 4096, (-2, 256, 16)), (17, 333, 1000, (-2, 40, 4)), (32, 4096, 2048, (-2, 256, 8)),
+    (25, 50, 1200, (-2, 9, 5))])
 def test_gemm_skinny(m, n, k, shape, out_dtype):
     x = randn(m, k, dtype=torch.bfloat16, seed=30, scale=0.5)
     w = randn(n, k, dtype=torch.bfloat16, seed=31, scale=0.5)
@@ -698,7 +699,8 @@ def test_gemm_skinny(m, n, k, shape, out_dtype):
 @pytest.mark.parametrize("m,n,k,shape,ksplit", [(8, 4096, 4096, (-1, 4, 4), 4), (1, 100, 12288, (-1, 4, 4), 4),
                                                 (16, 333, 1000, (-1, 8, 2), 2), (5, 64, 2560, (-1, 4, 4), 3),
                                                 (3, 48, 1000, (-1, 2, 2), 4), (8, 4096, 4096, (-2, 512, 4), 4),
-                                                (16, 130, 3000, (-2, 10, 4), 3), (2, 64, 12288, (-2, 30, 16), 3)])
+                                                (16, 130, 3000, (-2, 10, 4), 3), (2, 64, 12288, (-2, 30, 16), 3),
+                                                (32, 4096, 4096, (-2, 256, 4), 4), (20, 136, 5120, (-2, 33, 5), 4)])
 def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
     """Partial products [ksplit, M, N] in float: part s covers its own columns only, and the
     ordered sum is the product."""

@@ -26,7 +26,8 @@ def acceptable(m, n, k, silu, plan):
         return "more than 64 rows"
     kind, a, b = shape
     if kind == -2:
-        if m > 16 or b not in K.STAY_PIECES or not (256 * b * (parts - 1) < k <= 256 * b * parts) or a < 1:
+        if (m > 16 and (m > 32 or b > 8)) or b not in K.STAY_PIECES or a < 1 or \
+                not (256 * b * (parts - 1) < k <= 256 * b * parts):
             return "staying blocks that do not cover the inner size"
     elif kind == -1:
         phases = -(-k // (a * b * 32))
@@ -59,6 +60,7 @@ def test_plans_at_the_sizes_they_were_measured_at():
     assert plan(64, 4096, 12288, partial_ok=True) == (K.TILE64, 4)              # down_proj at 64 rows
     assert plan(64, 5120, 17408, partial_ok=True) == (K.TILE64, 3)              # 80 tiles of 64 rows: 3 groups fill 256 units
     assert plan(64, 4096, 4096, partial_ok=True) is None                        # short inner size: the library's
+    assert plan(32, 4096, 4096, partial_ok=True) == ((-2, 256, 4), 4)           # two row tiles of x in registers
     assert plan(12, 5120, 17408, partial_ok=True) == ((-2, 256, 17), 4)         # where the library collapses
     assert plan(8, 1024, 3072, partial_ok=True)[1] == 3                         # 6 phases do not share out to 4 groups
     assert plan(8, 4096, 4100) is None                                          # inner size no multiple of 8
