@@ -44,6 +44,7 @@ class RequestCache:
     hashes: list = field(default_factory=list)     # chain hashes of the full pages hashed so far (full group)
     num_cached_tokens: int = 0                     # tokens taken over from the prefix cache at start
     versions: list = field(default_factory=list)   # per group: bumped whenever the table changes
+    serial: int = 0                                # unique per start: a request id used again gets a new one
 
     @property
     def context_len(self) -> int:
@@ -65,6 +66,7 @@ class CacheManager:
         self.prefix_cache = bool(enable_prefix_cache and only_full and not has_state and self.groups)
         self.hit_tokens = 0
         self.new_slots: list = []   # slots assigned since the engine last zeroed state rows
+        self._starts = 0            # requests started so far (the next one's serial)
 
     # ---- queries
     def has(self, request_id) -> bool:
@@ -108,7 +110,8 @@ class CacheManager:
         if request_id in self.requests:
             raise KeyError(f"request {request_id!r} already started")
         rc = RequestCache(request_id, self.slots.acquire(), tables=[[] for _ in self.groups],
-                          versions=[0] * len(self.groups))
+                          versions=[0] * len(self.groups), serial=self._starts)
+        self._starts += 1
         self.new_slots.append(rc.slot)
         self.requests[request_id] = rc
         if self.prefix_cache and prompt is not None and len(prompt) > 1:
@@ -159,9 +162,13 @@ class CacheManager:
     def block_table(self, request_id, group: int) -> list:
         return self.requests[request_id].tables[group]
 
-    def table_version(self, request_id, group: int) -> int:
-        """Changes whenever the request's block table of this group does."""
-        return self.requests[request_id].versions[group]
+    def table_signature(self, request_id, group: int) -> tuple:
+        """Equal for two moments only if the block table of this group is the same one with the
+        same content: (serial of the start, version of the table).  A request id that is finished
+        and started again has another serial, so a copy of its old table is never taken for the
+        new one."""
+        rc = self.requests[request_id]
+        return (rc.serial, rc.versions[group])
 
     def slot(self, request_id) -> int:
         return self.requests[request_id].slot

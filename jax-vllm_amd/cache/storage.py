@@ -57,7 +57,8 @@ def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs:
                         f"window of {other.window} has already given back")
                 mem.k_pages, mem.v_pages, mem.group, mem.writes = owner.k_pages, owner.v_pages, owner.group, False
         if p.state is not None:
-            mem.state = torch.zeros((max_num_seqs, *p.state.shape), dtype=_STATE_DTYPES[p.state.dtype], device=device)
+            # one row per slot and a spare one that belongs to no request
+            mem.state = torch.zeros((max_num_seqs + 1, *p.state.shape), dtype=_STATE_DTYPES[p.state.dtype], device=device)
         memories.append(mem)
     return memories
 

@@ -1,6 +1,6 @@
 from .engine import EngineConfig, canonical_dtype
 from .errors import ConfigError
-from .model import Qwen3Config, read_config_json
+from .model import config_value, read_config_json
 from .registry import (
     Architecture,
     architecture_name,
@@ -11,6 +11,6 @@ from .registry import (
 )
 
 __all__ = [
-    "EngineConfig", "canonical_dtype", "ConfigError", "Qwen3Config", "read_config_json", "Architecture",
+    "EngineConfig", "canonical_dtype", "ConfigError", "config_value", "read_config_json", "Architecture",
     "architecture_name", "get_architecture", "register_architecture", "resolve", "supported_architectures",
 ]

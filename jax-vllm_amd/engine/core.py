@@ -67,7 +67,7 @@ class _DecodeGraph:
         self.host[a:b] = np.arange(rb + 1, dtype=np.int32)
         a, b = self.offsets["rows"]
         self.host[a:b] = np.arange(rb, dtype=np.int32)
-        self.row_signature = [[None] * rb for _ in range(n_groups)]   # (request, table version) per table row
+        self.row_signature = [[None] * rb for _ in range(n_groups)]   # the cache manager's table signature per row
         self.dev = torch.zeros(at, dtype=torch.int32, device=device)
         self.graph = None
         self.logits = None
@@ -83,6 +83,9 @@ class _DecodeGraph:
         return self.dev[a:b]
 
     def context(self, page_size: int, max_kv_len: int) -> StepContext:
+        """The context the launches are recorded with: device views of the fixed buffers; on the
+        host side only what holds for every replay (one token per row, an upper bound of the
+        context lengths, no slot ids)."""
         rb = self.rb
         return StepContext(
             num_tokens=rb, num_requests=rb, positions=self.dev_segment("positions"),
@@ -91,7 +94,7 @@ class _DecodeGraph:
             block_tables=[self.dev_segment(f"table{g}").view(rb, self.widths[g]) for g in range(self.n_groups)],
             slot_mappings=[self.dev_segment(f"slot_mapping{g}") for g in range(self.n_groups)],
             page_size=page_size, q_lens_host=[1] * rb, context_lens_host=[max_kv_len - 1] * rb,
-            slot_ids_host=[0] * rb, max_q_len=1, max_kv_len=max_kv_len,
+            slot_ids_host=None, max_q_len=1, max_kv_len=max_kv_len, captured=True,
         )
 
 
@@ -115,6 +118,11 @@ class EngineCore:
         self.kv_bytes_per_token = cache_bytes_per_token(self.plan, self.dtype)
         self._graphs: dict = {}
         self._max_graph_batch = min(config.max_num_seqs, 256)
+        # decode steps are recorded and replayed only if every part of the model has declared that
+        # it takes the step's values from the device (a part that plans on the host would replay
+        # the recorded step's plan for other requests)
+        self._replayable = model.replayable()
+        self._spare_slot = config.max_num_seqs     # the state row of rows that pad a captured step
         self.graph_replays = 0
 
     # ---- requests
@@ -160,7 +168,7 @@ class EngineCore:
 
     # ---- decode-only steps as replayed HIP graphs
     def _graphable(self, entries) -> bool:
-        if not self.config.use_hip_graphs or len(entries) > self._max_graph_batch:
+        if not self.config.use_hip_graphs or not self._replayable or len(entries) > self._max_graph_batch:
             return False
         return all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
 
@@ -184,8 +192,9 @@ class EngineCore:
         seg = g.segment
         reqs = [cache.requests[e.request_id] for e in entries]
         ctx_lens = [rc.context_len for rc in reqs]
-        for name in ("tokens", "positions", "ctx", "slots"):
+        for name in ("tokens", "positions", "ctx"):
             seg(host, name)[r:] = 0
+        seg(host, "slots")[r:] = self._spare_slot
         seg(host, "tokens")[:r] = [int(e.tokens[0]) for e in entries]
         seg(host, "positions")[:r] = ctx_lens
         seg(host, "ctx")[:r] = ctx_lens
@@ -198,7 +207,7 @@ class EngineCore:
             bt = seg(host, f"table{gi}").reshape(rb, widths[gi])
             sig = g.row_signature[gi]
             for i, rc in enumerate(reqs):
-                s = (rc.request_id, rc.versions[gi])
+                s = (rc.serial, rc.versions[gi])     # the serial, not the id: an id may be used again
                 if sig[i] != s:
                     t = rc.tables[gi]
                     bt[i, :len(t)] = t

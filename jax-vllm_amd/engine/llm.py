@@ -1,16 +1,15 @@
 """The Python entry point: an engine object with ``add_request / step / has_work`` and a
 blocking ``generate``, plus module-level functions in the reference's own manner
 (``make_driver``, ``add_request(driver, ...)``, ``step(driver)``, ``has_work(driver)``,
-``start / stream / stop`` for the loop in a thread of its own, ``prewarm``:
-``jllm/engine/engine.py:63-233``; the canonical loop is ``tests/_greedy.py:34-43``).
-Tokens in, tokens out: tokenisers are not part of the engine.
+``prewarm``: ``jllm/engine/engine.py:63-208``; the canonical loop is
+``tests/_greedy.py:34-43``).  The engine is stepped by its caller, in the caller's thread;
+the reference's background thread and per-request queues belong to its server and are not
+built.  Tokens in, tokens out: tokenisers are not part of the engine.
 """
 from __future__ import annotations
 
-import queue
-import threading
 from pathlib import Path
-from typing import Iterator, Mapping, Optional, Sequence, Union
+from typing import Mapping, Optional, Sequence, Union
 
 from ..config.engine import EngineConfig
 from ..sampling.keys import draw_key
@@ -32,13 +31,7 @@ class Engine:
         self._run, self._sample = run, sample
         self.vocab_size = vocab_size
         self._next_id = 0
-        self.requests: dict = {}
-        # background use (start / stream / stop): one lock for everything that touches the scheduler
-        self._wake = threading.Condition(threading.RLock())
-        self._thread: Optional[threading.Thread] = None
-        self._stopping = False
-        self._loop_error: Optional[BaseException] = None
-        self._streams: dict = {}
+        self.requests: dict = {}     # waiting and running requests by id; a finished one leaves with its last event
 
     # ---- the reference's loop: add_request / has_work / step
     def add_request(self, prompt_ids: Sequence[int], sampling: Optional[SamplingParams] = None,
@@ -49,16 +42,11 @@ class Engine:
                 raise ValueError(f"token id {t} outside the vocabulary [0, {self.vocab_size})")
         if sp.max_new_tokens < 1:
             raise ValueError("max_new_tokens must be at least 1")
-        with self._wake:
-            self._raise_if_failed()
-            rid = self._next_id
-            req = Request(request_id=rid, prompt_ids=[int(t) for t in prompt_ids], sampling=sp, arrival_step=arrival_step)
-            self.scheduler.add(req)
-            self._next_id += 1
-            self.requests[rid] = req
-            if self._thread is not None:
-                self._streams[rid] = queue.Queue()
-                self._wake.notify_all()
+        rid = self._next_id
+        req = Request(request_id=rid, prompt_ids=[int(t) for t in prompt_ids], sampling=sp, arrival_step=arrival_step)
+        self.scheduler.add(req)
+        self._next_id += 1
+        self.requests[rid] = req
         return rid
 
     def has_work(self) -> bool:
@@ -66,11 +54,8 @@ class Engine:
 
     def step(self) -> list:
         """One scheduler iteration: schedule, run the mixed batch, sample, finish.  Returns the
-        ``StepEvent`` of every token emitted."""
-        with self._wake:
-            return self._step()
-
-    def _step(self) -> list:
+        ``StepEvent`` of every token emitted.  The event that finishes a request carries the
+        request (prompt, output, counters); the engine keeps nothing of it afterwards."""
         out = self.scheduler.schedule()
         if not out.items:
             return []
@@ -106,86 +91,18 @@ class Engine:
             finished = self.scheduler.advance(item, tok)
             if tok is not None:
                 self.stats.emitted_tokens += 1
-                events.append(StepEvent(item.request.request_id, int(tok), finished))
+                events.append(StepEvent(item.request.request_id, int(tok), finished,
+                                        item.request if finished else None))
+            if finished:
+                self.requests.pop(item.request.request_id, None)
         return events
 
     def abort_all(self) -> None:
         """Drop every waiting and running request and give back what they hold."""
-        with self._wake:
-            self.scheduler.waiting.clear()
-            for req in list(self.scheduler.running):
-                self.scheduler.finish(req)
-            self.requests.clear()
-
-    # ---- background use, in the reference's manner (``jllm/engine/engine.py:134-154, 171-233``)
-    def start(self) -> None:
-        """Run the loop in a thread of its own: requests added from now on are stepped there and
-        their events are handed to ``stream``.  The thread sleeps while there is no work."""
-        with self._wake:
-            if self._thread is not None and self._thread.is_alive():
-                return
-            self._stopping, self._loop_error = False, None
-            self._thread = threading.Thread(target=self._loop, name="engine-loop", daemon=True)
-            self._thread.start()
-
-    def stop(self, join: bool = True) -> None:
-        with self._wake:
-            self._stopping = True
-            self._wake.notify_all()
-            thread = self._thread
-        if join and thread is not None:
-            thread.join()
-            with self._wake:
-                self._thread = None
-
-    def stream(self, request_id: int) -> Iterator[StepEvent]:
-        """The events of one request added after ``start``, as they are produced, up to and with
-        the one that finishes it.  Raises what the loop raised if it died."""
-        with self._wake:
-            q = self._streams.get(request_id)
-        if q is None:
-            raise KeyError(f"unknown or already drained request_id: {request_id}")
-        while True:
-            try:
-                ev = q.get(timeout=0.05)
-            except queue.Empty:
-                self._raise_if_failed()
-                if self._stopping and (self._thread is None or not self._thread.is_alive()):
-                    raise RuntimeError("engine stopped before the request finished") from None
-                continue
-            if ev is None:
-                self._raise_if_failed()
-                raise RuntimeError("engine stopped before the request finished")
-            yield ev
-            if ev.finished:
-                with self._wake:
-                    self._streams.pop(request_id, None)
-                    self.requests.pop(request_id, None)
-                return
-
-    def _raise_if_failed(self) -> None:
-        if self._loop_error is not None:
-            raise RuntimeError(f"the engine loop failed: {type(self._loop_error).__name__}: {self._loop_error}") \
-                from self._loop_error
-
-    def _loop(self) -> None:
-        try:
-            while True:
-                with self._wake:
-                    while not self._stopping and not self.scheduler.has_work():
-                        self._wake.wait()
-                    if self._stopping:
-                        return
-                    for ev in self._step():
-                        q = self._streams.get(ev.request_id)
-                        if q is not None:
-                            q.put(ev)
-        except BaseException as exc:   # handed to whoever streams or adds next
-            with self._wake:
-                self._loop_error = exc
-                self._stopping = True
-                for q in self._streams.values():
-                    q.put(None)
+        self.scheduler.waiting.clear()
+        for req in list(self.scheduler.running):
+            self.scheduler.finish(req)
+        self.requests.clear()
 
     # ---- blocking use
     def generate(self, prompts: Sequence[Sequence[int]],
@@ -195,15 +112,10 @@ class Engine:
         if sampling is None or isinstance(sampling, SamplingParams):
             sampling = [sampling or SamplingParams()] * len(prompts)
         arrival_steps = arrival_steps or [0] * len(prompts)
-        rids = [self.add_request(p, s, a) for p, s, a in zip(prompts, sampling, arrival_steps)]
+        reqs = [self.requests[self.add_request(p, s, a)] for p, s, a in zip(prompts, sampling, arrival_steps)]
         while self.has_work():
             self.step()
-        outs = [list(self.requests[r].output_ids) for r in rids]
-        with self._wake:
-            for r in rids:
-                del self.requests[r]
-                self._streams.pop(r, None)     # made if the background loop is running too
-        return outs
+        return [list(r.output_ids) for r in reqs]
 
 
 class LLM(Engine):
@@ -295,18 +207,6 @@ def has_work(driver: LLM) -> bool:
 
 def step(driver: LLM) -> list:
     return driver.step()
-
-
-def start(driver: LLM) -> None:
-    driver.start()
-
-
-def stop(driver: LLM, join: bool = True) -> None:
-    driver.stop(join)
-
-
-def stream(driver: LLM, request_id: int) -> Iterator[StepEvent]:
-    return driver.stream(request_id)
 
 
 def prewarm(driver: LLM) -> float:

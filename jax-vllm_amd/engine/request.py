@@ -45,6 +45,7 @@ class StepEvent:
     request_id: int
     token: int
     finished: bool
+    request: Optional[Request] = None   # with the finishing event only: the engine lets go of it there
 
 
 @dataclass

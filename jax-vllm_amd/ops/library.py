@@ -71,11 +71,26 @@ def _core_sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
+def _own_headers(sources: list[Path]) -> list[Path]:
+    """The package's headers that these sources include, directly or through one another."""
+    found, todo = {}, list(sources)
+    while todo:
+        src = todo.pop()
+        for line in src.read_text().splitlines():
+            line = line.strip()
+            if line.startswith("#include \""):
+                header = (src.parent / line.split("\"")[1]).resolve()
+                if header.exists() and header not in found:
+                    found[header] = True
+                    todo.append(header)
+    return sorted(found)
+
+
 def _stamp(sources: list[Path], extra: str = "") -> str:
     h = hashlib.sha256()
     h.update(" ".join(HIPCC_FLAGS).encode())
     h.update(extra.encode())
-    for p in sources + sorted(CSRC.glob("*.h")):
+    for p in sources + _own_headers(sources):
         h.update(p.name.encode())
         h.update(p.read_bytes())
     return h.hexdigest()

@@ -11,10 +11,11 @@ from .spec import (
     StepContext,
     TensorSpec,
     build_part,
+    is_replayable,
     register_part,
 )
 
 __all__ = [
     "DecoderModel", "Layer", "RunMemoryPlan", "KVCacheSpec", "LayerMemory", "LayerRun", "LayerSpec", "ModelSpec",
-    "PartSpec", "StateSpec", "StepContext", "TensorSpec", "build_part", "register_part",
+    "PartSpec", "StateSpec", "StepContext", "TensorSpec", "build_part", "is_replayable", "register_part",
 ]

@@ -15,7 +15,8 @@ from typing import Optional
 import torch
 
 from ..ops import kernels as K
-from .spec import KVCacheSpec, LayerMemory, PartSpec, StepContext, TensorSpec, build_part, register_part
+from .spec import (KVCacheSpec, LayerMemory, PartSpec, StepContext, TensorSpec, build_part, is_replayable,
+                   register_part)
 
 
 class GroupedQueryAttention:
@@ -32,6 +33,13 @@ class GroupedQueryAttention:
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
 
     # ---- declarations
+    @property
+    def replayable(self) -> bool:
+        """The kernels take positions, lengths and tables from the device; the host plan of a
+        captured step (how many blocks share a request's keys) is made for the upper bound of
+        the context lengths and is right for every shorter one."""
+        return self.position is None or is_replayable(self.position)
+
     def tensors(self) -> dict:
         t = {
             "q_proj.weight": TensorSpec((self.nq * self.d, self.hidden_size)),

@@ -10,7 +10,7 @@ from __future__ import annotations
 
 import torch
 
-from .spec import PartSpec, build_part, register_part
+from .spec import PartSpec, build_part, is_replayable, register_part
 
 
 class PreNormBlock:
@@ -19,6 +19,10 @@ class PreNormBlock:
         self.mixer_norm = build_part("norm", norm)
         self.feed_forward_norm = build_part("norm", norm)
         self.names = (mixer_norm_name, feed_forward_norm_name)
+
+    @property
+    def replayable(self) -> bool:
+        return is_replayable(self.mixer_norm) and is_replayable(self.feed_forward_norm)
 
     def tensors(self) -> dict:
         out = {}

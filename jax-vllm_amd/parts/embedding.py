@@ -10,6 +10,8 @@ from .spec import TensorSpec, register_part
 
 
 class TokenEmbedding:
+    replayable = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.weight = None
@@ -28,6 +30,8 @@ class TokenEmbedding:
 
 
 class LinearHead:
+    replayable = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
         self.weight = None

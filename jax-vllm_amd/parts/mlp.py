@@ -12,6 +12,8 @@ from .spec import TensorSpec, register_part
 
 
 class GatedMLP:
+    replayable = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         if activation != "silu":
             raise ValueError(f"GatedMLP has kernels for 'silu' only, not {activation!r}")

@@ -12,7 +12,8 @@ from typing import Optional
 
 import torch
 
-from .spec import KVCacheSpec, LayerMemory, LayerSpec, ModelSpec, StateSpec, StepContext, TensorSpec, build_part
+from .spec import (KVCacheSpec, LayerMemory, LayerSpec, ModelSpec, StateSpec, StepContext, TensorSpec, build_part,
+                   is_replayable)
 
 
 class Layer:
@@ -106,6 +107,15 @@ class DecoderModel:
             mixer = self.layers[run.layer].mixer
             plan.append(RunMemoryPlan(i, run.layer, mixer.cache_spec(), mixer.state_spec(), run.cache_of))
         return plan
+
+    def replayable(self) -> bool:
+        """Whether every part that runs in a step has declared that its launches may be recorded
+        once and replayed (see ``parts.spec.is_replayable``)."""
+        parts = [self.embedding, self.final_norm, self.head]
+        for run in self.spec.schedule:
+            layer = self.layers[run.layer]
+            parts += [layer.mixer, layer.feed_forward, layer.block]
+        return all(is_replayable(p) for p in parts)
 
     # ---- one step
     def forward(self, token_ids: torch.Tensor, ctx: StepContext, memories: list, logit_rows: torch.Tensor):

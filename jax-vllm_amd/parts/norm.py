@@ -14,6 +14,8 @@ from .spec import TensorSpec, register_part
 
 
 class RMSNorm:
+    replayable = True
+
     def __init__(self, size: int, eps: float):
         self.size, self.eps = int(size), float(eps)
         self.weight = None

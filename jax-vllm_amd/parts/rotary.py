@@ -17,6 +17,8 @@ from .spec import register_part
 
 
 class RotaryEncoding:
+    replayable = True      # the table is computed on the device from the step's positions
+
     def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None, interleaved: bool = False):
         self.head_dim = int(head_dim)
         self.theta = float(theta)

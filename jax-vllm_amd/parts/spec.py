@@ -65,7 +65,8 @@ class LayerMemory:
     k_pages [pages, kv_heads, page_size, head_dim], v_pages [pages, kv_heads, head_dim,
     page_size] (transposed), or None; ``group`` says which
     block table / slot mapping of the step applies; ``writes`` is False for a run that reads
-    another run's cache.  ``state`` is [slots, *shape] or None.
+    another run's cache.  ``state`` is [slots + 1, *shape] or None; its last row belongs to no
+    request (rows that pad a captured step point there).
     """
 
     k_pages: Optional[torch.Tensor] = None
@@ -81,6 +82,13 @@ class StepContext:
 
     Tokens of all requests are flattened, request after request.  Device tensors are
     int32.  Host mirrors are Python lists for parts that plan work on the host.
+
+    ``captured``: the launches of this step are recorded once and replayed for later steps
+    with other requests in the same rows.  Then only the device tensors carry the step's
+    values: ``q_lens_host`` is exact (ones), ``context_lens_host`` holds an upper bound for
+    every row, ``slot_ids_host`` is None, and rows that pad the batch have the null page in
+    their tables, slot mapping -1 and the spare state slot (the last row of ``LayerMemory.state``).
+    Only models whose parts all declare ``replayable = True`` are ever run this way.
     """
 
     num_tokens: int
@@ -95,15 +103,25 @@ class StepContext:
     page_size: int
     q_lens_host: list                  # [R] tokens of each request in this step
     context_lens_host: list            # [R]
-    slot_ids_host: list                # [R]
+    slot_ids_host: Optional[list]      # [R]; None in a captured step
     max_q_len: int = 1
     max_kv_len: int = 1
     extras: dict = field(default_factory=dict)   # per-step results of kernels, shared by parts of one kind
     plans: dict = field(default_factory=dict)    # per-step work lists built on the host and uploaded
+    captured: bool = False
 
     @property
     def decode_only(self) -> bool:
         return self.max_q_len == 1
+
+
+def is_replayable(part) -> bool:
+    """Whether a part's ``forward`` may be recorded once and replayed for later steps: it reads
+    the step's values (positions, lengths, tables, slots) from the context's device tensors only
+    and uses the host mirrors at most as upper bounds for planning.  A part says so with a class
+    or instance attribute ``replayable = True``; a part that says nothing is taken to plan on the
+    host and its model's decode steps are never captured."""
+    return bool(getattr(part, "replayable", False))
 
 
 # --------------------------------------------------------------------------- registry of parts

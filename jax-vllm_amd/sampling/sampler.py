@@ -31,4 +31,10 @@ class Sampler:
             temp = torch.tensor(list(temperatures), dtype=torch.float32, device=self.device)
             key = torch.tensor(list(keys), dtype=torch.int64, device=self.device)
             out = K.sample(logits, temp, key)
-        return out.tolist()
+        ids = out.tolist()
+        vocab = logits.shape[1]
+        bad = [i for i, t in enumerate(ids) if not 0 <= t < vocab]
+        if bad:
+            # the kernel answers "no token" (the vocabulary size) for a row without any comparable value
+            raise FloatingPointError(f"logits row(s) {bad} of {m} hold no finite maximum (NaN): no token can be chosen")
+        return ids

@@ -3,7 +3,11 @@
 Reference: ``jllm/model/weights.py:21-37`` (all shards in sorted order, a later shard wins
 on a duplicate name, every tensor cast to the engine's type) and ``:161-170`` (the model
 is chosen by ``architectures[0]``).  Unlike the reference, names and shapes are checked
-before anything is copied, and all problems are reported in one error.
+before anything is copied, and all problems are reported in one error.  Like the reference
+(whose dictionary of tensors is simply never asked for the other names), tensors that the
+model does not use are no problem by themselves: they are named once on standard error and
+left alone, unless ``strict`` asks for an error; an error for another reason lists them too,
+since a missing tensor and an unexpected one are often the same tensor under two names.
 
 Types on the device: tensors of role "matrix" take the compute type (bfloat16 or float32),
 role "vector" is float32 (16-bit values widen exactly, 32-bit values stay as stored),
@@ -11,6 +15,7 @@ role "table" is int32.
 """
 from __future__ import annotations
 
+import sys
 from pathlib import Path
 
 import torch
@@ -57,8 +62,10 @@ def target_dtype(role: str, compute_dtype: torch.dtype) -> torch.dtype:
     raise ValueError(f"unknown tensor role {role!r}")
 
 
-def check_against_specs(where, specs: dict, ignored: set, available: dict) -> None:
-    """``available``: name -> (dtype, shape) found in the checkpoint."""
+def check_against_specs(where, specs: dict, ignored: set, available: dict, strict: bool = False) -> list:
+    """``available``: name -> (dtype, shape) found in the checkpoint.  Raises one ``WeightsError``
+    for all missing tensors, wrong shapes and wrong types (and, if ``strict``, for tensors the
+    model does not use); returns the names of the unused tensors otherwise."""
     missing = [n for n in specs if n not in available]
     unexpected = [n for n in available if n not in specs and n not in ignored]
     wrong_shape, wrong_type = [], []
@@ -71,12 +78,14 @@ def check_against_specs(where, specs: dict, ignored: set, available: dict) -> No
         is_float = dtype.is_floating_point
         if (ts.role == "table") == is_float:
             wrong_type.append((name, str(dtype).replace("torch.", ""), "integer" if ts.role == "table" else "floating"))
-    if missing or unexpected or wrong_shape or wrong_type:
+    if missing or wrong_shape or wrong_type or (strict and unexpected):
         raise WeightsError(where, missing, unexpected, wrong_shape, wrong_type)
+    return sorted(unexpected)
 
 
-def load_model(folder, dtype: str = "bfloat16", device="cuda") -> tuple:
-    """(bound DecoderModel, typed config) of a model folder."""
+def load_model(folder, dtype: str = "bfloat16", device="cuda", strict: bool = False) -> tuple:
+    """(bound DecoderModel, typed config) of a model folder.  ``strict``: tensors in the folder
+    that the model does not use are an error instead of a line on standard error."""
     folder = Path(folder)
     arch, cfg, _ = resolve(folder)
     model = DecoderModel(arch.build_spec(cfg))
@@ -87,7 +96,10 @@ def load_model(folder, dtype: str = "bfloat16", device="cuda") -> tuple:
     for shard in shards:  # a later shard wins
         for name, entry in shard.entries.items():
             owner[name], available[name] = shard, entry
-    check_against_specs(folder, specs, ignored, available)
+    unused = check_against_specs(folder, specs, ignored, available, strict)
+    if unused:
+        print(f"[jax_vllm_amd] {folder}: {len(unused)} tensor(s) not used by the model: " + ", ".join(unused),
+              file=sys.stderr, flush=True)
     tensors = {}
     for name, ts in specs.items():
         src = owner[name].tensor(name)

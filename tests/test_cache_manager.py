@@ -210,3 +210,32 @@ def test_random_orders_keep_every_page_accounted_for(seed):
         m.finish(rid)
     m.check_invariants()
     assert all(g.pool.num_free == 24 for g in m.groups) and m.slots.num_free == 5
+
+
+def test_table_signature_tells_a_restarted_id_from_its_earlier_life():
+    """A copy of a block table is valid as long as the table's signature is unchanged.  The
+    signature changes with every change of the table and differs between two starts of the
+    same request id, also when both lives made the same number of changes."""
+    m = CacheManager([("full",), ("window", 8)], 4, 12, 3, enable_prefix_cache=False)
+    seen = set()
+    for life in range(3):
+        m.start("r")
+        m.reserve("r", 8)                  # two pages at once: one change
+        sig = m.table_signature("r", 0)
+        assert sig not in seen
+        seen.add(sig)
+        assert m.table_signature("r", 0) == sig            # asking changes nothing
+        m.commit("r", list(range(8)))
+        assert m.table_signature("r", 0) == sig            # the full group's table did not change
+        m.reserve("r", 1)
+        assert m.table_signature("r", 0) != sig
+        m.commit("r", [1])
+        w = m.table_signature("r", 1)
+        m.reserve("r", 3)
+        m.commit("r", [1, 2, 3])           # position 12 next: the window group gives its first page back
+        assert m.block_table("r", 1)[0] == 0 and m.table_signature("r", 1) != w
+        m.finish("r")
+    # two requests never share a signature either
+    m.start("a"), m.start("b")
+    m.reserve("a", 4), m.reserve("b", 4)
+    assert m.table_signature("a", 0) != m.table_signature("b", 0)

@@ -4,7 +4,8 @@ import json
 import pytest
 import torch
 
-from jax_vllm_amd.config import ConfigError, EngineConfig, Qwen3Config, resolve, supported_architectures
+from jax_vllm_amd.config import ConfigError, EngineConfig, resolve, supported_architectures
+from jax_vllm_amd.models.qwen3 import Qwen3Config
 from jax_vllm_amd.parts import DecoderModel, LayerRun, ModelSpec
 from jax_vllm_amd.weights.loader import WeightsError, check_against_specs
 from jax_vllm_amd.weights.random_init import write_random_model
@@ -139,6 +140,39 @@ def test_weight_errors_list_everything_at_once():
     assert "wrong shape: model.layers.0.mlp.up_proj.weight is [64, 128], the model needs [128, 64]" in msg
     assert "wrong type: model.embed_tokens.weight is stored as int64" in msg
     assert e.value.missing == ["model.layers.1.self_attn.k_norm.weight", "model.norm.weight"]
+
+
+def test_unused_tensors_are_named_and_tolerated_unless_strict(tmp_path, capsys):
+    """jllm/model/weights.py:21-37 reads every tensor of the folder into a dictionary and the
+    model asks it only for the names it uses: leftovers (a stored inv_freq buffer, an extra
+    head) do not stop a load.  Here they are named on standard error; ``strict`` refuses them;
+    a missing tensor stays an error and the error lists the unused ones too."""
+    from jax_vllm_amd.weights.loader import load_model
+
+    folder = write_random_model(tmp_path / "m", TINY_A["config"], seed=0, std=0.02, norm_std=0.02)
+    f = SafetensorsFile(folder / "model.safetensors")
+    items = [(n, tuple(shape), dtype, (lambda n=n: f.tensor(n))) for n, (dtype, shape) in f.entries.items()]
+    extra = "model.layers.0.self_attn.rotary_emb.inv_freq"
+    items.append((extra, (8,), torch.float32, lambda: torch.arange(8, dtype=torch.float32)))
+    write_safetensors(folder / "model.safetensors.new", items)
+    f.close()
+    (folder / "model.safetensors.new").rename(folder / "model.safetensors")
+    model, cfg = load_model(folder, "float32", "cpu")
+    err = capsys.readouterr().err
+    assert "1 tensor(s) not used by the model: " + extra in err
+    assert model.layers[0].mixer.w_qkv.shape == (4 * 16 + 2 * 2 * 16, 64)
+    with pytest.raises(WeightsError, match="unexpected tensors \\(1\\): " + extra):
+        load_model(folder, "float32", "cpu", strict=True)
+    # without strict the checker hands the names back and raises only for real problems
+    arch, c, _ = resolve(TINY_A["config"])
+    specs = DecoderModel(arch.build_spec(c)).tensor_specs()
+    available = {k: (torch.bfloat16, tuple(v.shape)) for k, v in specs.items()}
+    available[extra] = (torch.float32, (8,))
+    assert check_against_specs("x", specs, set(), available) == [extra]
+    del available["model.norm.weight"]
+    with pytest.raises(WeightsError) as e:
+        check_against_specs("x", specs, set(), available)
+    assert e.value.missing == ["model.norm.weight"] and e.value.unexpected == [extra]
 
 
 def test_model_spec_rejects_bad_schedules():

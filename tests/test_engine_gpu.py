@@ -55,6 +55,40 @@ def test_greedy_generation_workload_a(folders, dtype):
     assert out == got[1]
 
 
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_command_line_generates_what_the_plain_implementation_does(folders, dtype, tmp_path, capsys):
+    """``main`` from the options to the printed token ids (the reference's entry is
+    jllm/server.py:245-306; tokens in, tokens out here): prompts from --prompt-ids and from a
+    file, prewarm on (the default), one line of ids per prompt on standard output."""
+    from jax_vllm_amd.engine import cli
+
+    cfg, w = plain_of(folders["C"])
+    rng = np.random.default_rng(23)
+    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (3, 32, 45)]
+    (tmp_path / "p.txt").write_text("\n".join(" ".join(map(str, p)) for p in prompts[1:]) + "\n")
+    code = cli.main(["--model-path", str(folders["C"]), "--prompt-ids", ",".join(map(str, prompts[0])),
+                     "--prompt-file", str(tmp_path / "p.txt"), "--max-new-tokens", "8", "--dtype", dtype,
+                     "--block-size", str(TINY_C["page_size"]), "--max-model-len", "128", "--max-num-seqs", "3",
+                     "--max-num-batched-tokens", "40", "--stats"])
+    assert code == 0
+    cap = capsys.readouterr()
+    lines = [l for l in cap.out.splitlines() if l.strip()]
+    assert len(lines) == 3 and "prewarmed in" in cap.err and "EngineStats(" in cap.err
+    got = [[int(t) for t in l.split()] for l in lines]
+    assert [len(g) for g in got] == [8, 8, 8]
+    if dtype == "fp32":
+        assert got == [P.greedy_generate(w, cfg, p, 8) for p in prompts]
+    for p, g in zip(prompts, got):
+        check_tokens_follow(dtype, cfg, w, p, g)
+    # an eos id ends a request early and is printed
+    code = cli.main(["--model-path", str(folders["C"]), "--prompt-ids", " ".join(map(str, prompts[0])), "--max-new-tokens", "8",
+                     "--dtype", "fp32", "--block-size", "32", "--max-model-len", "64", "--no-prewarm", "--no-hip-graphs",
+                     "--eos-id", str(P.greedy_generate(w, cfg, prompts[0], 8)[2])])
+    out = [int(t) for t in capsys.readouterr().out.split()]
+    want = P.greedy_generate(w, cfg, prompts[0], 8)
+    assert code == 0 and out == want[:want.index(want[2]) + 1]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_prewarm_leaves_the_engine_as_it_was(folders, dtype):
     """``prewarm`` (the reference's ``jllm/engine/engine.py:182-208``) captures the decode step for
@@ -94,26 +128,32 @@ def test_prewarm_leaves_the_engine_as_it_was(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_streaming_from_a_background_loop(folders, dtype):
-    """The engine stepped in a thread of its own (``start`` / ``stream`` / ``stop``) gives the tokens
-    of the blocking loop, captured decode steps included."""
-    from jax_vllm_amd import LLM, SamplingParams, start, stop, stream
+def test_request_ids_used_again_after_prewarm_read_their_own_pages(folders, dtype):
+    """``prewarm`` gives its warm-up requests the ids 0, 1, ... and hands the same ids to the first
+    real requests.  A captured decode step keeps a copy of every row's block table and rewrites
+    it only when the table's signature changes; a real request whose table has the same number of
+    reserves as the warm-up request of the same id (a prompt of exactly one or two pages; a
+    prompt cut into two portions by the token budget) must still get its own pages into the row.
+    The pool is drawn on first, so the real requests' pages are not the warm-up's."""
+    from jax_vllm_amd import LLM, SamplingParams
 
-    cfg, w = plain_of(folders["A"])
-    rng = np.random.default_rng(12)
-    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (4, 19, 33)]
-    llm = LLM(folders["A"], dtype=dtype, block_size=TINY_A["page_size"], max_num_seqs=3, max_model_len=64,
-              max_num_batched_tokens=32)
-    sp = SamplingParams(max_new_tokens=10)
-    want = llm.generate(prompts, sp)
-    start(llm)
-    rids = [llm.add_request(p, sp) for p in prompts]
-    got = [[ev.token for ev in stream(llm, r)] for r in rids]
-    stop(llm)
-    assert got == want
-    for p, g in zip(prompts, got):
-        check_tokens_follow(dtype, cfg, w, p, g)
-    assert llm.generate(prompts[:1], sp) == want[:1]          # and the blocking loop works again afterwards
+    cfg, w = plain_of(folders["B"])
+    ps = TINY_B["page_size"]
+    rng = np.random.default_rng(31)
+    opts = dict(dtype=dtype, block_size=ps, max_num_seqs=4, max_model_len=160, max_num_batched_tokens=64,
+                enable_prefix_cache=False)
+    for lengths in ([ps, 2 * ps, 3 * ps], [100, ps]):          # 100 tokens under a budget of 64: two portions
+        llm = LLM(folders["B"], **opts)
+        llm.prewarm()
+        # hold a few pages so that the next requests get other pages than the warm-up requests had
+        held = [llm.core.cache.groups[0].pool.allocate() for _ in range(7)]
+        prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in lengths]
+        got = llm.generate(prompts, SamplingParams(max_new_tokens=10))
+        assert llm.stats.graph_replays > 0
+        for p, g in zip(prompts, got):
+            check_tokens_follow(dtype, cfg, w, p, g)
+        llm.core.cache.groups[0].pool.release(held)
+        llm.core.cache.check_invariants()
 
 
 def test_temperature_generation_workload_b_is_cut_independent(folders):
@@ -138,15 +178,26 @@ def test_temperature_generation_workload_b_is_cut_independent(folders):
     assert b.generate(prompts, sp) == got
     c = LLM(folders["B"], max_num_seqs=3, max_num_batched_tokens=7, num_blocks=1 + 9, **base)
     assert c.generate(prompts, sp) == got
-    # sampled tokens are plausible under the plain distribution and not simply greedy
+    # not simply greedy; and each token is the one that the same draw picks from the *plain*
+    # logits: the draw of request r's i-th token has the key of (seed, r, i) and depends on nothing
+    # else, so the sampling kernel applied to the plain implementation's last row must give the
+    # engine's token (that the kernel's draws follow softmax(logits / T) is the kernel tests' subject)
+    from jax_vllm_amd.ops import kernels as K
+    from jax_vllm_amd.sampling import draw_key
+
     greedy = LLM(folders["B"], max_num_seqs=4, max_num_batched_tokens=2048, **base).generate(prompts, SamplingParams(max_new_tokens=20))
     assert greedy != got
-    for p, g in zip(prompts, got):
+    rows, keys, flat = [], [], []
+    for r, (p, g) in enumerate(zip(prompts, got)):
         seq = list(p)
-        for t in g:
-            prob = P.softmax_temperature(P.forward(w, cfg, seq)[-1], 0.8)[t].item()
-            assert prob > 1e-5
+        for i, t in enumerate(g):
+            rows.append(P.forward(w, cfg, seq)[-1])
+            keys.append(draw_key(7, r, i))
+            flat.append(t)
             seq.append(t)
+    picked = K.sample(torch.stack(rows).cuda(), torch.full((len(rows),), 0.8, device="cuda"),
+                      torch.tensor(keys, dtype=torch.int64, device="cuda")).tolist()
+    assert picked == flat
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -211,6 +262,81 @@ def test_replayed_decode_steps_equal_eager_steps(folders, dtype):
     for i, got in zip(range(20, 40), outs[id(graph)]):
         live = [r for r, t in reqs.items() if i < len(t)]
         check_logits(dtype, got.numpy(), np.stack([expected[r][i] for r in live]), what=f"position {i}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_replayed_decode_steps_of_many_requests(folders, dtype):
+    """Captured decode steps with 20 and then 40 live requests (rows of the step: 24 and 48, of
+    which the last are padding), while requests end and the rows are handed to others: every
+    row's logits against the plain implementation.  The replays' padding rows read the null page
+    and store nothing."""
+    cfg, w = plain_of(folders["B"])
+    rng = np.random.default_rng(17)
+    lengths = [int(n) for n in rng.integers(20, 56, size=40)]
+    reqs = {f"r{i}": rng.integers(0, cfg["vocab_size"], size=n).tolist() for i, n in enumerate(lengths)}
+    expected = {r: P.forward(w, cfg, t).numpy() for r, t in reqs.items()}
+    core = make_core(folders["B"], dtype, 16, pages=200, seqs=48, graphs=True)
+    fed = {}
+
+    def admit(names, first):
+        for r in names:
+            core.start_request(r)
+            fed[r] = first
+        core.run([entry(r, reqs[r][:first], []) for r in names])
+
+    def decode_all():
+        live = [r for r in fed if fed[r] < len(reqs[r])]
+        out = core.run([entry(r, reqs[r][fed[r]:fed[r] + 1], [0]) for r in live]).cpu().numpy()
+        check_logits(dtype, out, np.stack([expected[r][fed[r]] for r in live]), what=f"{len(live)} live")
+        for r in live:
+            fed[r] += 1
+            if fed[r] == len(reqs[r]):
+                core.finish_request(r)
+        return len(live)
+
+    names = list(reqs)
+    admit(names[:20], 12)
+    widths = [decode_all() for _ in range(6)]
+    assert widths == [20] * 6
+    admit(names[20:], 15)
+    while any(fed[r] < len(reqs[r]) for r in fed):
+        widths.append(decode_all())
+    assert 40 in widths and any(17 <= x <= 24 for x in widths[6:])    # rows of 48 and of 24, rows handed on
+    assert {k[0] for k in core._graphs} >= {24, 48} and core.graph_replays >= 20
+    core.cache.check_invariants()
+    assert core.cache.num_free_pages() == 200
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_replayed_decode_steps_with_a_window_group(folders, dtype):
+    """A model with a full-attention layer group and a windowed one, decoded through captured
+    steps: the window group's table rows change as pages are given back (its signature moves,
+    the captured step's copy of the row must follow)."""
+    cfg, w = plain_of(folders["B"])
+    schedule = [(0, None), (1, None), (2, None)]
+    windows = {1: 20}
+    model = custom_model(folders["B"], dtype, schedule, windows)
+    core = make_core(None, dtype, 16, pages=30, seqs=3, model=model, graphs=True)
+    assert core.group_keys == [("full",), ("window", 20)]
+    rng = np.random.default_rng(19)
+    reqs = {r: rng.integers(0, cfg["vocab_size"], size=n).tolist() for r, n in (("a", 120), ("b", 90))}
+    want = {r: P.forward_scheduled(w, cfg, t, schedule, windows).numpy() for r, t in reqs.items()}
+    got = {r: [] for r in reqs}
+    for r in reqs:
+        core.start_request(r)
+    out = core.run([entry("a", reqs["a"][:30]), entry("b", reqs["b"][:7])]).cpu().numpy()
+    got["a"].append(out[:30]), got["b"].append(out[30:])
+    fed = {"a": 30, "b": 7}
+    while any(fed[r] < len(reqs[r]) for r in reqs):
+        live = [r for r in reqs if fed[r] < len(reqs[r])]
+        out = core.run([entry(r, reqs[r][fed[r]:fed[r] + 1]) for r in live]).cpu().numpy()
+        for i, r in enumerate(live):
+            got[r].append(out[i:i + 1])
+            fed[r] += 1
+    assert core.graph_replays >= 80
+    for r in reqs:
+        check_logits(dtype, np.concatenate(got[r]), want[r], what=r)
+    assert core.cache.block_table("a", 1)[:5] == [0] * 5        # the window has moved on
 
 
 # ------------------------------------------------------------------ long decoding, first tokens
@@ -503,7 +629,9 @@ def test_schedule_repeats_a_layer_shares_a_cache_and_windows(folders, dtype):
 class RunningMeanMixer:
     """A toy token mixer with state of its own, defined here and registered from here: its
     output at a token is a projection of the mean of all inputs of the request up to and
-    including that token.  State per request: the running sum (float).  No pages."""
+    including that token.  State per request: the running sum (float).  No pages.  It plans on
+    the host (reads the context's host mirrors) and says nothing about replaying, so the engine
+    never records its steps."""
 
     def __init__(self, hidden_size: int):
         self.hidden_size = hidden_size
@@ -537,18 +665,37 @@ class RunningMeanMixer:
         return out
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype):
+class RunningMeanMixerOnDevice(RunningMeanMixer):
+    """The same function, but a step of single tokens takes slots and positions from the
+    context's device tensors only, so it may be recorded and replayed: it declares so."""
+
+    replayable = True
+
+    def forward(self, x, ctx, mem):
+        if not ctx.decode_only:
+            assert not ctx.captured
+            return super().forward(x, ctx, mem)
+        slots = ctx.slot_ids.long()
+        sums = mem.state[slots] + x.float()
+        mem.state[slots] = sums                  # rows that pad a recorded step write the spare row
+        counts = (ctx.positions + 1).float()[:, None]
+        return ((sums / counts).to(x.dtype) @ self.w.t()).to(x.dtype)
+
+
+def toy_state_model(dtype, mixer_kind):
+    """(bound model, float weights by name) of a four-run model: toy mixer, attention, toy mixer,
+    and the first layer once more (its weights shared, a state of its own)."""
     from jax_vllm_amd.config import register_architecture, resolve
     from jax_vllm_amd.parts import DecoderModel, LayerRun, LayerSpec, ModelSpec, PartSpec, register_part
     from jax_vllm_amd.weights.loader import TORCH_DTYPES, target_dtype
 
     register_part("mixer", "running_mean", RunningMeanMixer)
-    hidden, vocab, inter = 48, 120, 96
+    register_part("mixer", "running_mean_on_device", RunningMeanMixerOnDevice)
+    hidden, vocab, inter = TOY_STATE["hidden"], TOY_STATE["vocab"], TOY_STATE["inter"]
     norm = PartSpec("rmsnorm", {"size": hidden, "eps": 1e-5})
     att = PartSpec("gqa_attention", dict(hidden_size=hidden, num_heads=3, num_kv_heads=1, head_dim=16, qk_norm_eps=1e-5,
                                          position=PartSpec("rotary", {"head_dim": 16, "theta": 1e4})))
-    toy = PartSpec("running_mean", {"hidden_size": hidden})
+    toy = PartSpec(mixer_kind, {"hidden_size": hidden})
     ffn = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter})
 
     def build(_cfg):
@@ -569,26 +716,46 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype):
     w = {n: ((0.2 * torch.randn(ts.shape, generator=g)) if ts.role == "matrix" else 1 + 0.1 * torch.randn(ts.shape, generator=g))
          .to(torch.bfloat16).float() for n, ts in model.tensor_specs().items()}
     model.bind({n: v.cuda().to(target_dtype(model.tensor_specs()[n].role, compute)) for n, v in w.items()}, compute)
-    core = make_core(None, dtype, 8, pages=24, seqs=3, model=model)
+    return model, w
+
+
+TOY_STATE = dict(hidden=48, vocab=120, inter=96)
+
+
+def toy_state_plain(w, tokens):
+    """The toy model written out whole: no state, a cumulative mean over the sequence."""
+    t = len(tokens)
+    pos = torch.arange(t)
+    c = dict(num_heads=3, num_kv_heads=1, head_dim=16, rms_norm_eps=1e-5, rope_theta=1e4)
+    h = w["emb.weight"][torch.tensor(tokens)]
+    for i in (0, 1, 2, 0):
+        x = P.rms_norm(w[f"l{i}.input_layernorm.weight"], 1e-5, h)
+        if i == 1:
+            a = P.attention_block(w, "l1.mix", c, x, pos)
+        else:
+            a = (torch.cumsum(x, 0) / torch.arange(1, t + 1)[:, None]) @ w[f"l{i}.mix.proj.weight"].T
+        h = h + a
+        m = P.rms_norm(w[f"l{i}.post_attention_layernorm.weight"], 1e-5, h)
+        h = h + P.swiglu(w[f"l{i}.ffn.gate_proj.weight"], w[f"l{i}.ffn.up_proj.weight"], w[f"l{i}.ffn.down_proj.weight"], m)
+    return (P.rms_norm(w["norm.weight"], 1e-5, h) @ w["emb.weight"].T).numpy()
+
+
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs-on"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype, graphs):
+    """With HIP graphs switched on as well: the mixer plans on the host and has not declared
+    itself replayable, so every step runs eagerly with its true slots."""
+    hidden, vocab = TOY_STATE["hidden"], TOY_STATE["vocab"]
+    model, w = toy_state_model(dtype, "running_mean")
+    core = make_core(None, dtype, 8, pages=24, seqs=3, model=model, graphs=graphs)
     assert [p.state is not None for p in core.plan] == [True, False, True, True]
     assert not core.cache.prefix_cache                      # state forbids taking pages over
-    assert [m.state.shape for m in core.memories if m.state is not None] == [(3, hidden)] * 3
+    assert not model.replayable()
+    # one row per slot and the spare row
+    assert [m.state.shape for m in core.memories if m.state is not None] == [(4, hidden)] * 3
 
     def plain(tokens):
-        t = len(tokens)
-        pos = torch.arange(t)
-        c = dict(num_heads=3, num_kv_heads=1, head_dim=16, rms_norm_eps=1e-5, rope_theta=1e4)
-        h = w["emb.weight"][torch.tensor(tokens)]
-        for i in (0, 1, 2, 0):
-            x = P.rms_norm(w[f"l{i}.input_layernorm.weight"], 1e-5, h)
-            if i == 1:
-                a = P.attention_block(w, "l1.mix", c, x, pos)
-            else:
-                a = (torch.cumsum(x, 0) / torch.arange(1, t + 1)[:, None]) @ w[f"l{i}.mix.proj.weight"].T
-            h = h + a
-            m = P.rms_norm(w[f"l{i}.post_attention_layernorm.weight"], 1e-5, h)
-            h = h + P.swiglu(w[f"l{i}.ffn.gate_proj.weight"], w[f"l{i}.ffn.up_proj.weight"], w[f"l{i}.ffn.down_proj.weight"], m)
-        return (P.rms_norm(w["norm.weight"], 1e-5, h) @ w["emb.weight"].T).numpy()
+        return toy_state_plain(w, tokens)
 
     rng = np.random.default_rng(6)
     reqs = {r: rng.integers(0, vocab, size=n).tolist() for r, n in (("a", 40), ("b", 23), ("c", 31))}
@@ -596,7 +763,8 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype):
     got = {r: [] for r in reqs}
     for r in reqs:
         core.start_request(r)
-    cuts = [[("a", 7)], [("a", 2), ("b", 9)], [("b", 1), ("c", 31), ("a", 1)], [("a", 30), ("b", 13)]]
+    cuts = [[("a", 7)], [("a", 2), ("b", 9)], [("b", 1), ("c", 31), ("a", 1)], [("a", 20), ("b", 8)]]
+    cuts += [[("a", 1), ("b", 1)]] * 5 + [[("a", 1)]] * 5       # the tails one by one: steps a graph engine would record
     for step in cuts:
         es = [entry(r, reqs[r][fed[r]:fed[r] + n]) for r, n in step]
         out = core.run(es).cpu().numpy()
@@ -605,6 +773,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype):
             got[r].append(out[at:at + n])
             at += n
             fed[r] += n
+    assert core.graph_replays == 0 and not core._graphs
     for r in reqs:
         assert fed[r] == len(reqs[r])
         check_logits(dtype, np.concatenate(got[r]), plain(reqs[r]), what=r)
@@ -613,6 +782,51 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(folders, dtype):
     core.start_request("d")
     out = core.run([entry("d", reqs["c"])]).cpu().numpy()
     check_logits(dtype, out, plain(reqs["c"]), what="d after b")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_state_on_the_device_is_recorded_and_replayed(dtype):
+    """The same toy model with a mixer that declares ``replayable``: its decode steps are recorded
+    and replayed.  Three live requests make a step of four rows: the padding row writes the spare
+    state row, never a request's; requests end and their slots are taken again from zero."""
+    vocab = TOY_STATE["vocab"]
+    model, w = toy_state_model(dtype, "running_mean_on_device")
+    assert model.replayable()
+    core = make_core(None, dtype, 8, pages=40, seqs=4, model=model, graphs=True)
+    rng = np.random.default_rng(7)
+    reqs = {r: rng.integers(0, vocab, size=n).tolist() for r, n in (("a", 40), ("b", 33), ("c", 36), ("d", 30), ("e", 25))}
+    want = {r: toy_state_plain(w, t) for r, t in reqs.items()}
+    fed, got = {}, {r: [] for r in reqs}
+
+    def admit(r, n):
+        core.start_request(r)
+        got[r].append(core.run([entry(r, reqs[r][:n])]).cpu().numpy())
+        fed[r] = n
+
+    def decode():
+        live = [r for r in fed if fed[r] < len(reqs[r])]
+        out = core.run([entry(r, reqs[r][fed[r]:fed[r] + 1]) for r in live]).cpu().numpy()
+        for i, r in enumerate(live):
+            got[r].append(out[i:i + 1])
+            fed[r] += 1
+            if fed[r] == len(reqs[r]):
+                core.finish_request(r)
+        return len(live)
+
+    admit("a", 9), admit("b", 17), admit("c", 5)
+    for _ in range(16):
+        assert decode() == 3                    # four rows, one of them padding
+    admit("d", 11)                               # slot 3
+    while fed["b"] < len(reqs["b"]):
+        decode()
+    admit("e", 8)                                # b's slot again: zeroed
+    while any(fed[r] < len(reqs[r]) for r in fed):
+        decode()
+    assert core.graph_replays >= 30
+    for r in reqs:
+        check_logits(dtype, np.concatenate(got[r]), want[r], what=r)
+    spare = [m.state[-1] for m in core.memories if m.state is not None]
+    assert any(float(s.abs().max()) > 0 for s in spare)      # the padding rows did write there
 
 
 class TopOneExperts:

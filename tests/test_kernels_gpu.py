@@ -398,6 +398,21 @@ def test_greedy_is_argmax_lowest_index_on_ties():
     assert out[2].item() == 100 and out[4].item() == 776
 
 
+def test_a_row_without_a_maximum_is_an_error_not_a_token():
+    """A row of NaN logits has no winner: the kernel answers with the vocabulary size and the
+    sampler above it raises at once, instead of handing on a token that no table has."""
+    from jax_vllm_amd.sampling.sampler import Sampler
+
+    logits = randn(3, 300, seed=21)
+    logits[1] = float("nan")
+    assert K().sample(logits).tolist()[1] == 300
+    with pytest.raises(FloatingPointError, match=r"row\(s\) \[1\] of 3"):
+        Sampler(logits.device).sample(logits, [0.0, 0.0, 0.0], [1, 2, 3])
+    logits[1] = 0.0
+    logits[1, 7] = float("nan")                       # one NaN among numbers never wins
+    assert Sampler(logits.device).sample(logits, [0.0, 0.0, 0.0], [1, 2, 3])[1] == 0
+
+
 def test_temperature_sampling_matches_softmax():
     v, n, temp = 11, 20000, 0.8
     logits1 = randn(1, v, seed=21, scale=1.5)

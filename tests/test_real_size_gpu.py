@@ -1,6 +1,7 @@
 """The layer sizes of real models (Qwen3-8B: hidden 4096, 32/8 heads of 128, feed-forward
-12288, vocabulary 151936; and the 14B sizes: hidden 5120, 40/8 heads, feed-forward 17408) with two
-layers of random weights: the 32-bit path and the bfloat16
+12288, vocabulary 151936; the 14B sizes: hidden 5120, 40/8 heads, feed-forward 17408; the 32B
+sizes: hidden 5120, 64/8 heads, so that heads * head size = 8192 is not the width, feed-forward
+25600) with two layers of random weights: the 32-bit path and the bfloat16
 path against the plain implementation, whole, token by token, in portions and mixed.  These are
 the sizes at which the kernels' wide paths run (16-byte norm loads, the streaming matrix
 product's real shapes, a vocabulary that is no power of two, the 128-wide MFMA attention)."""
@@ -19,9 +20,12 @@ CONFIG = dict(architectures=["Qwen3ForCausalLM"], num_hidden_layers=2, hidden_si
 # the next size up: 5 query heads per kv head, a width of 5120 (inner sizes that are no multiple of
 # 4096: other organisations of the streaming products), a feed-forward of 17408
 CONFIG_14B = dict(CONFIG, hidden_size=5120, num_attention_heads=40, intermediate_size=17408)
+# 8 query heads per kv head; the attention's output is wider than the model (8192 against 5120), the
+# feed-forward's inner size is beyond what one block keeps of x: further branches of the products' plans
+CONFIG_32B = dict(CONFIG, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
 
 
-@pytest.fixture(scope="module", params=[CONFIG, CONFIG_14B], ids=["8b", "14b"])
+@pytest.fixture(scope="module", params=[CONFIG, CONFIG_14B, CONFIG_32B], ids=["8b", "14b", "32b"])
 def big(request):
     CONFIG = request.param
     from jax_vllm_amd.config import resolve

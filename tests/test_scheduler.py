@@ -210,10 +210,11 @@ def test_decode_without_a_page_preempts_the_newest_request():
     p0, p1 = list(range(9)), list(range(20, 29))
     a = eng.add_request(p0, SamplingParams(max_new_tokens=8))
     b = eng.add_request(p1, SamplingParams(max_new_tokens=8))
+    ra, rb = eng.requests[a], eng.requests[b]
     drain(eng)
     assert eng.stats.preemptions >= 1
-    assert eng.requests[b].num_preemptions >= 1 and eng.requests[a].num_preemptions == 0   # the newest yields
-    assert eng.requests[a].output_ids == expected(p0, 8) and eng.requests[b].output_ids == expected(p1, 8)
+    assert rb.num_preemptions >= 1 and ra.num_preemptions == 0   # the newest yields
+    assert ra.output_ids == expected(p0, 8) and rb.output_ids == expected(p1, 8)
     # the preempted request was recomputed from position 0: prompt and the tokens it had generated
     restarts = [s for s in core.steps for rid, c, n, _ in s if rid == b and c == 0]
     assert len(restarts) >= 2
@@ -225,10 +226,11 @@ def test_prompt_portion_is_shortened_or_postponed_when_pages_are_short():
                      enable_prefix_cache=False)
     a = eng.add_request(list(range(14)), SamplingParams(max_new_tokens=2))     # 4 pages
     b = eng.add_request(list(range(30, 44)), SamplingParams(max_new_tokens=2))  # wants 4, only 2 are free
+    ra, rb = eng.requests[a], eng.requests[b]
     drain(eng)
     assert core.steps[0] == [(a, 0, 14, [13])]                # b is not admitted: its first portion has no room
-    assert eng.requests[a].output_ids == expected(list(range(14)), 2)
-    assert eng.requests[b].output_ids == expected(list(range(30, 44)), 2)
+    assert ra.output_ids == expected(list(range(14)), 2)
+    assert rb.output_ids == expected(list(range(30, 44)), 2)
     assert eng.stats.preemptions == 0
 
 
@@ -274,43 +276,27 @@ def test_random_workloads_with_few_pages_finish_right(seed):
     assert core.cache.num_free_pages() == eng.config.usable_pages
 
 
-def test_background_loop_streams_what_the_blocking_loop_generates():
-    """``start`` / ``stream`` / ``stop`` (the reference's threaded use, jllm/engine/engine.py:134-233):
-    requests added while the loop runs in its own thread give the same tokens as ``generate``,
-    every stream ends with the finishing event, and the thread sleeps without work."""
-    prompts = [[1, 2, 3], list(range(40)), [7] * 17]
-    sp = SamplingParams(max_new_tokens=9)
-    blocking, _ = make(max_num_seqs=2, max_model_len=128, block_size=8, max_num_batched_tokens=16)
-    want = blocking.generate(prompts, sp)
-    eng, _ = make(max_num_seqs=2, max_model_len=128, block_size=8, max_num_batched_tokens=16)
-    eng.start()
-    eng.start()                                   # a second start changes nothing
-    rids = [eng.add_request(p, sp) for p in prompts]
-    got = []
-    for rid in reversed(rids):                    # drained in another order than they were added
-        events = list(eng.stream(rid))
-        assert [e.request_id for e in events] == [rid] * 9 and [e.finished for e in events] == [False] * 8 + [True]
-        got.append([e.token for e in events])
-    assert got[::-1] == want and not eng.has_work() and eng.requests == {}
-    with pytest.raises(KeyError):
-        next(eng.stream(rids[0]))                 # already drained
-    late = eng.add_request([5, 6], SamplingParams(max_new_tokens=3))     # the sleeping thread wakes up
-    assert len(list(eng.stream(late))) == 3
-    eng.stop()
-    assert eng._thread is None
-
-
-def test_background_loop_hands_its_failure_to_the_caller():
-    eng, core = make(max_num_seqs=2, max_model_len=64, block_size=8, max_num_batched_tokens=16)
-
-    def broken(entries, borrow=False):
-        raise ValueError("the step function broke")
-
-    eng._run = broken
-    eng.start()
-    rid = eng.add_request([1, 2, 3], SamplingParams(max_new_tokens=4))
-    with pytest.raises(RuntimeError, match="the step function broke"):
-        list(eng.stream(rid))
-    with pytest.raises(RuntimeError, match="engine loop failed"):
-        eng.add_request([4], SamplingParams(max_new_tokens=1))
-    eng.stop()
+def test_the_stepped_loop_hands_out_finished_requests_and_keeps_none():
+    """The reference's canonical loop (tests/_greedy.py:34-43 there): add_request, then step while
+    has_work, collecting events.  Every request's last event says finished and carries the
+    request; the engine's own table holds waiting and running requests only, so a long-lived
+    engine does not grow with the requests it has served."""
+    prompts = [[1, 2, 3], list(range(40)), [7] * 17, [9], list(range(50, 70))]
+    eng, core = make(max_num_seqs=2, max_model_len=128, block_size=8, max_num_batched_tokens=16)
+    rids = [eng.add_request(p, SamplingParams(max_new_tokens=5 + i)) for i, p in enumerate(prompts)]
+    assert sorted(eng.requests) == rids
+    tokens, done, peak = {r: [] for r in rids}, {}, 0
+    while eng.has_work():
+        for ev in eng.step():
+            assert ev.request_id not in done
+            tokens[ev.request_id].append(ev.token)
+            assert (ev.request is not None) == ev.finished
+            if ev.finished:
+                done[ev.request_id] = ev.request
+                assert ev.request_id not in eng.requests
+        peak = max(peak, len(eng.requests))
+    assert eng.requests == {} and sorted(done) == rids
+    for i, (rid, p) in enumerate(zip(rids, prompts)):
+        assert tokens[rid] == done[rid].output_ids == expected(p, 5 + i) and done[rid].prompt_ids == p
+    core.cache.check_invariants()
+    assert core.cache.num_free_pages() == eng.config.usable_pages
