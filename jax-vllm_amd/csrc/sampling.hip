@@ -6,6 +6,10 @@
 //     comes from a counter-based generator keyed by (key[r], i).  The draw depends on
 //     the row's key and logits only, not on the batch it is in.
 #include "common.h"
+#include "sampling.h"
+
+#include <mutex>
+#include <stdio.h>
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
   z += 0x9E3779B97F4A7C15ull;
@@ -92,6 +96,22 @@ sample_stage2_kernel(int* __restrict__ out, const float* __restrict__ part_v, co
 
 #define SAMPLE_MAX_CHUNKS 64
 
+static int sample_launch(int* out, const float* logits, long long row_stride, int n_rows, int V,
+                         const float* temperature, const unsigned long long* keys, void* scratch,
+                         hipStream_t stream) {
+  int chunks = (V + 4095) / 4096;  // at least 4096 columns per block
+  if (chunks > SAMPLE_MAX_CHUNKS) chunks = SAMPLE_MAX_CHUNKS;
+  const int chunk = (V + chunks - 1) / chunks;
+  float* pv = (float*)scratch;
+  int* pi = (int*)(pv + (long long)n_rows * SAMPLE_MAX_CHUNKS);
+  hipLaunchKernelGGL(sample_stage1_kernel, dim3(chunks, n_rows), dim3(256), 0, stream, pv, pi, logits, row_stride,
+                     V, chunk, temperature, keys);
+  int e = JV_LAUNCH_CHECK();
+  if (e) return e;
+  hipLaunchKernelGGL(sample_stage2_kernel, dim3(n_rows), dim3(64), 0, stream, out, pv, pi, chunks, V);
+  return JV_LAUNCH_CHECK();
+}
+
 // scratch: SAMPLE_MAX_CHUNKS * n_rows floats followed by as many ints (jv_sample_scratch_bytes)
 extern "C" long long jv_sample_scratch_bytes(int n_rows) { return (long long)n_rows * SAMPLE_MAX_CHUNKS * 8; }
 
@@ -100,15 +120,83 @@ extern "C" int jv_sample(int* out, const float* logits, long long row_stride, in
                          void* stream) {
   if (n_rows <= 0) return 0;
   if (V <= 0 || !scratch || n_rows > 65535) return (int)hipErrorInvalidValue;
-  int chunks = (V + 4095) / 4096;  // at least 4096 columns per block
-  if (chunks > SAMPLE_MAX_CHUNKS) chunks = SAMPLE_MAX_CHUNKS;
-  const int chunk = (V + chunks - 1) / chunks;
-  float* pv = (float*)scratch;
-  int* pi = (int*)(pv + (long long)n_rows * SAMPLE_MAX_CHUNKS);
-  hipLaunchKernelGGL(sample_stage1_kernel, dim3(chunks, n_rows), dim3(256), 0, (hipStream_t)stream, pv, pi,
-                     logits, row_stride, V, chunk, temperature, keys);
-  int e = JV_LAUNCH_CHECK();
+  return sample_launch(out, logits, row_stride, n_rows, V, temperature, keys, scratch, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same choice of tokens without a workspace from the caller: the stage-one winners go to a
+// fixed array in device memory that the library itself holds, on every GPU it runs on, until the
+// process ends (JV_SAMPLE_NOALLOC_MAX_ROWS * 64 chunks * 8 bytes = 512 KiB).  Nothing is allocated
+// or freed here or by anything this calls.  Stage one writes every (row, chunk) entry that stage
+// two reads, so nothing has to start at zero and what an earlier call left does not matter.  All
+// calls on one GPU share the array: two calls that overlap there (different streams, or graphs
+// replayed at the same time) race on it.
+static __device__ __align__(256) unsigned char sample_noalloc_scratch[JV_SAMPLE_NOALLOC_MAX_ROWS * SAMPLE_MAX_CHUNKS * 8];
+
+#define SAMPLE_NOALLOC_MAX_DEVICES 64
+// The array's address on each device.  In host code the array's name is only a stand-in for the
+// symbol; the address a kernel can use comes from hipGetSymbolAddress, and each GPU has its own.
+static void* sample_noalloc_ptr[SAMPLE_NOALLOC_MAX_DEVICES];
+static std::mutex sample_noalloc_mutex;
+static thread_local char sample_noalloc_error[256];
+
+extern "C" const char* jv_sample_noalloc_last_error(void) { return sample_noalloc_error; }
+
+// Resolves the array's address on the current device (once per device).  Returns 0 or a hipError_t.
+static int sample_noalloc_resolve(void** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    snprintf(sample_noalloc_error, sizeof sample_noalloc_error, "jv_sample_noalloc: hipGetDevice failed: %s",
+             hipGetErrorString(e));
+    return (int)e;
+  }
+  if (dev < 0 || dev >= SAMPLE_NOALLOC_MAX_DEVICES) {
+    snprintf(sample_noalloc_error, sizeof sample_noalloc_error,
+             "jv_sample_noalloc: device %d is beyond the %d devices this entry point keeps an address for", dev,
+             SAMPLE_NOALLOC_MAX_DEVICES);
+    return (int)hipErrorInvalidDevice;
+  }
+  std::lock_guard<std::mutex> lock(sample_noalloc_mutex);
+  if (!sample_noalloc_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(sample_noalloc_scratch));
+    if (e != hipSuccess || !p) {
+      snprintf(sample_noalloc_error, sizeof sample_noalloc_error,
+               "jv_sample_noalloc: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+    }
+    sample_noalloc_ptr[dev] = p;
+  }
+  *ptr = sample_noalloc_ptr[dev];
+  return 0;
+}
+
+extern "C" int jv_sample_noalloc_init(void) {
+  void* p = nullptr;
+  sample_noalloc_error[0] = 0;
+  return sample_noalloc_resolve(&p);
+}
+
+extern "C" int jv_sample_noalloc(int* out, const float* logits, long long row_stride, int n_rows, int V,
+                                 const float* temperature, const unsigned long long* keys, void* stream) {
+  sample_noalloc_error[0] = 0;
+  if (n_rows <= 0) return 0;
+  if (n_rows > JV_SAMPLE_NOALLOC_MAX_ROWS) {
+    snprintf(sample_noalloc_error, sizeof sample_noalloc_error,
+             "jv_sample_noalloc: %d rows exceed the maximum of %d that the fixed %d KiB array holds; "
+             "call it on slices of the rows or use jv_sample with a workspace", n_rows, JV_SAMPLE_NOALLOC_MAX_ROWS,
+             JV_SAMPLE_NOALLOC_MAX_ROWS * SAMPLE_MAX_CHUNKS * 8 / 1024);
+    return (int)hipErrorInvalidValue;
+  }
+  if (V <= 0 || !out || !logits || (temperature && !keys)) {
+    snprintf(sample_noalloc_error, sizeof sample_noalloc_error,
+             "jv_sample_noalloc: needs out, logits, a vocabulary of at least 1 and keys wherever temperatures are given");
+    return (int)hipErrorInvalidValue;
+  }
+  void* scratch = nullptr;
+  const int e = sample_noalloc_resolve(&scratch);
   if (e) return e;
-  hipLaunchKernelGGL(sample_stage2_kernel, dim3(n_rows), dim3(64), 0, (hipStream_t)stream, out, pv, pi, chunks, V);
-  return JV_LAUNCH_CHECK();
+  // from here on only the resolved address is used, never the array's name
+  return sample_launch(out, logits, row_stride, n_rows, V, temperature, keys, scratch, (hipStream_t)stream);
 }
