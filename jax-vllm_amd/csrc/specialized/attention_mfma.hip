@@ -19,7 +19,9 @@
 // Rows of a work item are the (query, head-in-group) pairs of one request and one kv head:
 // row m = query_index * G + head_in_group, G = q heads per kv head; any G works.
 //   prefill kernel: 128 rows per block (4 waves x 2 row tiles of 16; 64 rows for heads above 128), K/V tiles of 64 keys staged
-//                   in LDS and shared by the 4 waves; causal limit and window per row.
+//                   in LDS and shared by the 4 waves; causal limit and window per row.  Head sizes that are
+//                   multiples of 32 up to 128 have a kernel of their own instead (32x32x16 products, one tile
+//                   of 32 rows per wave, tiles straight from global memory into LDS): see JV_PREFILL32.
 //   decode kernel:  one query per request; each of the 4 waves streams its own 32-key tiles
 //                   straight from global memory into MFMA operands (no LDS), the waves'
 //                   partial (max, sum, acc) are merged in LDS; with num_splits > 1 several
@@ -31,6 +33,9 @@
 #error "compile with -DJV_HEAD_DIM=<head size>"
 #endif
 static_assert(JV_HEAD_DIM % 16 == 0 && JV_HEAD_DIM >= 16 && JV_HEAD_DIM <= 256, "head size");
+#if JV_HEAD_DIM % 32 == 0 && JV_HEAD_DIM <= 128
+#define JV_PREFILL32 1   // the prefill kernel with 32-row tiles is built, the one with 16-row tiles is not
+#endif
 
 constexpr int D = JV_HEAD_DIM;
 constexpr int NDT = D / 16;                // 16-wide tiles of the head dimension (output)
@@ -101,6 +106,7 @@ constexpr int NO_GAP = 0x7fffffff;
 #else
 #define PREFILL_OCCUPANCY
 #endif
+#ifndef JV_PREFILL32
 // PAGES: 1 = the page size is 8, 16, 32 or 64 (pages tile the 64 keys: a thread's slot in its
 // page is the same in every tile), 2 = a larger power of two, 0 = any other multiple of 8.
 template <int PAGES>
@@ -484,9 +490,420 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
   }
 }
 
+#endif  // !JV_PREFILL32
+
+// ------------------------------------------------------------------------------------ prefill, 32-row tiles
+// Head sizes that are multiples of 32 up to 128 take this kernel.  It reads the same work items
+// (two groups of 64 rows) but gives every wave ONE tile of 32 rows (waves 0, 1: first group,
+// waves 2, 3: second group) and multiplies with v_mfma_f32_32x32x16_bf16: a 16-byte fragment of K
+// or V^T read from LDS then feeds a product of 32 cycles, twice as much as with 16x16x32 tiles
+// of a single row tile, and the kernel lives on the LDS rate (128 B/clk for 16-byte reads, half
+// of that for 8-byte ones).  What makes every LDS access one of 16 bytes:
+//   * S^T accumulators of a 32-key block hold, for the lane halves h = 0, 1, product rows
+//     8i + 4h + j (i, j < 4).  Product row 8i + 4h + j is fed with key 16(i/2) + 8h + 4(i%2) + j of
+//     the block (only a lane's LDS read address changes), so the two accumulator quads i = 2s,
+//     2s + 1 of a lane are the 8 CONSECUTIVE keys 16s + 8h .. + 7: exactly the B operand of
+//     O^T += V^T P^T for keys 16s .. 16s + 15, whose A operand is then a plain 16-byte read of
+//     V^T[d][16s + 8h ..].
+//   * both tiles are stored in 16-byte chunks whose position inside each 256-byte line is
+//     xor-ed with the line number: reads of 32 rows at one column and writes of whole rows are
+//     both conflict-free (measured).
+// Tiles are double-buffered in LDS: one barrier per 64 keys.
+#ifdef JV_PREFILL32
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+// a wave in a burst of products goes first: the other wave of its SIMD (of the compute unit's other block) then
+// does its softmax meanwhile instead of contending for the matrix unit
+#define JV_PRIO(x) __builtin_amdgcn_s_setprio(x)
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+constexpr int NQS = D / 16;                // contraction steps of S^T = K Q^T
+constexpr int NDB = D / 32;                // 32-row blocks of O^T
+constexpr int CPK = D / 8;                 // 16-byte chunks of a key row
+constexpr int TBL32 = 1024;                // page-table entries a block keeps in LDS at a time
+constexpr int PCS = BN * CPK / 256;        // 16-byte pieces of a K tile (and of a V^T tile) per thread
+constexpr bool KB_ADDS = (32 * CPK / 16) % 16 == 0;   // the second key block's chunks are the first's plus a constant
+__device__ __forceinline__ int swizzle(int q) { return q ^ ((q >> 4) & 15); }   // chunk index -> chunk position
+
+template <int PAGES>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) attn_prefill32_kernel(AttnArgs p) {
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[2][BN * D];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[2][D * BN];
+  // FAST: pages of 16 keys and a head size that is a power of two.  Every load instruction of a wave
+  // then lies in ONE page, whose number is a scalar read straight from the request's table, and a
+  // lane's address is that page's base plus a constant of the lane.
+  constexpr bool FAST = PAGES == 16;
+  static_assert(!FAST || (64 % CPK == 0), "the fast path needs whole keys per load instruction");
+  __shared__ int page_ids[FAST ? 1 : TBL32];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // a scalar: branches on it are uniform
+  const int l32 = lane & 31, h = lane >> 5;
+  const int g = blockIdx.x % p.nkv, item = blockIdx.x / p.nkv;
+  const int r = p.work[3 * item];
+  const int G = p.nq / p.nkv, P = FAST ? 16 : p.page_size;
+  const PageSplit ps{P, PAGES == 0 ? -1 : (FAST ? 4 : p.page_shift)};
+  const int q_start = p.cu_seqlens[r], q_len = p.cu_seqlens[r + 1] - q_start;
+  const int ctx = p.context_lens[r];
+  const int M = q_len * G;
+  const int* gtable = p.block_tables + (long long)r * p.table_stride;
+
+  // ---- the block's two groups: keys [begin, end) that some row of a group sees
+  int blk_begin[2], blk_end[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int m0 = p.work[3 * item + 1 + t];
+    blk_begin[t] = blk_end[t] = 0;
+    if (m0 >= 0 && m0 < M) {
+      const int last_row = (M < m0 + 64 ? M : m0 + 64) - 1;
+      blk_end[t] = ctx + last_row / G + 1;
+      if (p.window > 0) {
+        blk_begin[t] = ctx + m0 / G - p.window + 1;
+        if (blk_begin[t] < 0) blk_begin[t] = 0;
+      }
+    }
+  }
+  // ---- this wave's tile of 32 rows and this lane's row
+  const int m0 = p.work[3 * item + 1 + (wave >> 1)];
+  const int wave_first = m0 + (wave & 1) * 32;
+  const bool wave_live = m0 >= 0 && wave_first < M;
+  const int wave_last = (M < wave_first + 32 ? M : wave_first + 32) - 1;
+  const int wave_kv_end = wave_live ? ctx + wave_last / G + 1 : 0;
+  const int wave_min_pos = ctx + wave_first / G;
+  int wave_kv_begin = 0, wave_full_begin = 0;
+  if (p.window > 0 && wave_live) {
+    wave_kv_begin = wave_min_pos - p.window + 1;
+    if (wave_kv_begin < 0) wave_kv_begin = 0;
+    wave_full_begin = ctx + wave_last / G - p.window + 1;
+    if (wave_full_begin < 0) wave_full_begin = 0;
+  }
+  const int row = wave_first + l32;
+  const bool row_ok = wave_live && row < M;
+  const int qi = row_ok ? row / G : 0, hg = row_ok ? row - qi * G : 0;
+  const int pos = ctx + qi;
+  bf16x8 qf[NQS];                          // B operand: row l32, head elements 16 ks + 8 h .. + 7
+  {
+    const bf16_t* qrow = p.q + (long long)(q_start + qi) * p.q_row_stride + (long long)(g * G + hg) * D + h * 8;
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int ks = 0; ks < NQS; ++ks) qf[ks] = row_ok ? *(const bf16x8*)(qrow + ks * 16) : zero8;
+  }
+
+  // ---- the tiles the block walks (the union of the two groups' ranges; a window may leave a gap)
+  int j_first, kv_end, gap_from = NO_GAP, gap_to = NO_GAP;
+  {
+    int b0 = blk_begin[0] / BN * BN, e0 = blk_end[0];
+    int b1 = blk_begin[1] / BN * BN, e1 = blk_end[1];
+    if (e1 <= b1) { b1 = b0; e1 = e0; }
+    if (e0 <= b0) { b0 = b1; e0 = e1; }
+    if (b1 < b0) { int x = b0; b0 = b1; b1 = x; x = e0; e0 = e1; e1 = x; }
+    j_first = b0;
+    kv_end = e0 > e1 ? e0 : e1;
+    const int e0_up = (e0 + BN - 1) / BN * BN;
+    if (b1 > e0_up) { gap_from = e0_up; gap_to = b1; }
+  }
+  auto next_tile = [&](int j0) { return j0 + BN == gap_from ? gap_to : j0 + BN; };
+  if (kv_end <= j_first) return;                    // nothing to do (the same in every thread)
+
+  const int last_page = ps.index(kv_end - 1);
+  int seg_first = 0;
+  auto load_table = [&](int j) {                    // called by all threads, between barriers
+    seg_first = ps.index(j);
+    int n = last_page - seg_first + 1;
+    if (n > TBL32) n = TBL32;
+    for (int i = tid; i < n; i += 256) page_ids[i] = gtable[seg_first + i];
+  };
+  if (!FAST) {
+    load_table(j_first);
+    __syncthreads();
+  }
+
+  // ---- pieces of a tile.  A tile goes from global memory straight into LDS (no registers between):
+  // instruction i of wave w fills the 64 chunk positions (4i + w) * 64 .. + 63 of the buffer, lane l the
+  // position (4i + w) * 64 + l, so the lane asks for the chunk that belongs there (both swizzles are
+  // their own inverses).  K is stored key by key, 256-byte lines xor-ed with the line number.  V^T is
+  // stored d row by d row of 64 keys in the general path; in the fast path page by page, [page][d][2
+  // chunks], positions xor-ed with the lowest bit of the line number: a wave's 64 chunks are then 32
+  // whole d rows of one page, 1 KB in one piece, and the reads of 32 d at one key chunk stay
+  // conflict-free (8 d rows a line, neighbouring lines swap their even and odd positions).
+  const unsigned page_stride = (unsigned)p.nkv * (unsigned)P * (unsigned)D;   // elements; the host checks it fits
+  auto v_swizzle = [&](int q) { return FAST ? (q ^ ((q >> 4) & 1)) : swizzle(q); };
+  int k_off[PCS], v_off[PCS], k_key[PCS], v_key[PCS];
+#pragma unroll
+  for (int i = 0; i < PCS; ++i) {
+    const int pos = (4 * i + wave) * 64 + lane;
+    const int q = swizzle(pos);
+    const int key = q / CPK, dc = q - key * CPK;
+    k_key[i] = key;
+    k_off[i] = (g * P + (PAGES != 0 && PAGES != 2 ? (key & (P - 1)) : 0)) * D + dc * 8;
+    const int qv = v_swizzle(pos);
+    if (FAST) {
+      const int pg = qv / (2 * D), d = (qv - pg * 2 * D) >> 1, c = qv & 1;
+      v_key[i] = pg * 16 + c * 8;
+      v_off[i] = (g * D + d) * 16 + c * 8;
+    } else {
+      const int d = qv / (BN / 8), kc = qv - d * (BN / 8);
+      v_key[i] = kc * 8;
+      v_off[i] = (g * D + d) * P + (PAGES == 1 ? ((kc * 8) & (P - 1)) : 0);
+    }
+  }
+  typedef const __attribute__((address_space(1))) void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
+  // Nothing here looks at a loaded value.  A piece past the last key reads the same slot of the last
+  // page (allocated memory): K there is masked by position, V is zeroed in LDS by fix_tail.
+  // fast path: the PCS pages of this wave's instructions for the tile at j0, as scalars from the
+  // table (read-only for the kernel's life, hence the constant address space: scalar loads that
+  // nothing else waits on).  They are asked for one tile before the tile's loads are issued.
+  typedef const __attribute__((address_space(4))) int* ctable_t;
+  const ctable_t ctable = (ctable_t)(unsigned long long)gtable;
+  auto pages_of = [&](int j0, unsigned (&pg)[PCS]) {
+#pragma unroll
+    for (int i = 0; i < PCS; ++i) {
+      int pi = (j0 >> 4) + (((4 * i + wave) * 64) / (2 * D));   // first key of the instruction, (4i + w) * 64 / CPK, over 16
+      if (pi > last_page) pi = last_page;
+      pg[i] = (unsigned)ctable[pi];
+    }
+  };
+  auto fetch_fast = [&](int b, const unsigned (&pg)[PCS]) {
+#pragma unroll
+    for (int i = 0; i < PCS; ++i) {
+      const unsigned long long base = (unsigned long long)pg[i] * page_stride;   // scalar
+      __builtin_amdgcn_global_load_lds((gptr_t)(p.k_pages + base + (unsigned)k_off[i]),
+                                       (lptr_t)&Ks[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((gptr_t)(p.v_pages + base + (unsigned)v_off[i]),
+                                       (lptr_t)&Vs[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
+    }
+  };
+  auto fetch = [&](int j0, int b) {
+    int j_hi = j0 + BN - 1;
+    if (j_hi > kv_end - 1) j_hi = kv_end - 1;
+    if (ps.index(j_hi) - seg_first >= TBL32) {      // same decision in every thread
+      __syncthreads();
+      load_table(j0);
+      __syncthreads();
+    }
+    const int tile_page = ps.index(j0) - seg_first, end_page = last_page - seg_first;
+#pragma unroll
+    for (int i = 0; i < PCS; ++i) {
+      int pi, off = k_off[i];
+      if (PAGES == 1) {
+        pi = tile_page + (k_key[i] >> ps.shift);
+      } else {
+        const int j = j0 + k_key[i];
+        pi = ps.index(j) - seg_first;
+        off += ps.slot(j) * D;
+      }
+      if (pi > end_page) pi = end_page;
+      const unsigned page = (unsigned)page_ids[pi];
+      __builtin_amdgcn_global_load_lds((gptr_t)(p.k_pages + ((unsigned long long)page * page_stride + (unsigned)off)),
+                                       (lptr_t)&Ks[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < PCS; ++i) {
+      int pi, off = v_off[i];
+      if (PAGES == 1) {
+        pi = tile_page + (v_key[i] >> ps.shift);
+      } else {
+        const int j = j0 + v_key[i];
+        pi = ps.index(j) - seg_first;
+        off += ps.slot(j);
+      }
+      if (pi > end_page) pi = end_page;
+      const unsigned page = (unsigned)page_ids[pi];
+      __builtin_amdgcn_global_load_lds((gptr_t)(p.v_pages + ((unsigned long long)page * page_stride + (unsigned)off)),
+                                       (lptr_t)&Vs[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
+    }
+  };
+  // V entries of keys at or past kv_end become zeros (their probabilities are zeros, and zero times a
+  // stale NaN is not): every thread cleans the pieces it asked for, once they have arrived.
+  auto fix_tail = [&](int j0, int b) {
+#pragma unroll
+    for (int i = 0; i < PCS; ++i) {
+      const int j = j0 + v_key[i];
+      if (j + 8 > kv_end) {
+        bf16x8* at = (bf16x8*)&Vs[b][((4 * i + wave) * 64 + lane) * 8];
+        bf16x8 v = *at;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (j + e >= kv_end) v[e] = (bf16_t)0.f;
+        *at = v;
+      }
+    }
+  };
+  auto arrived = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+
+  // ---- LDS read addresses (elements).  K: product row l32 = 8i + 4hh + j reads key 16(i/2) + 8hh + 4(i%2) + j.
+  const int krow = ((l32 >> 4) << 4) | (((l32 >> 2) & 1) << 3) | (((l32 >> 3) & 1) << 2) | (l32 & 3);
+  auto k_read = [&](int kb, int ks) { return swizzle((kb * 32 + krow) * CPK + 2 * ks + h) * 8; };
+  int kr[NQS];
+#pragma unroll
+  for (int ks = 0; ks < NQS; ++ks) kr[ks] = k_read(0, ks);
+  int vr[BN / 16];                                  // d = l32 (+ 32 db: adds a constant), keys 16 s + 8 h .. + 7
+#pragma unroll
+  for (int s = 0; s < BN / 16; ++s)
+    vr[s] = (FAST ? v_swizzle(s * 2 * D + l32 * 2 + h) : swizzle(l32 * (BN / 8) + 2 * s + h)) * 8;
+  constexpr int V_DB = FAST ? 32 * 2 * 8 : 32 * BN;  // elements from one block of 32 d to the next
+  // the key that element e = 4i + j of a 32-key block's accumulator belongs to, less the block's first
+  auto acc_key = [&](int e) { return 16 * (e >> 3) + 8 * h + 4 * ((e >> 2) & 1) + (e & 3); };
+
+  float m_run = -INFINITY, m_ref = -INFINITY, l_lane = 0.f;
+  f32x16 acc[NDB];
+#pragma unroll
+  for (int db = 0; db < NDB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
+
+  auto multiply = [&](int j0, int b) {
+    const bf16_t* Kb = Ks[b];
+    const bf16_t* Vb = Vs[b];
+    f32x16 s[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
+    // S^T: fragments are read two steps ahead of their products
+    bf16x8 kf[3][2];
+    auto read_k = [&](int ks, bf16x8 (&f)[2]) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+        f[kb] = *(const bf16x8*)(Kb + (KB_ADDS ? kr[ks] + kb * 32 * D : k_read(kb, ks)));
+    };
+    read_k(0, kf[0]);
+    if (NQS > 1) read_k(1, kf[1]);
+    JV_PRIO(1);
+#pragma unroll
+    for (int ks = 0; ks < NQS; ++ks) {
+      if (ks + 2 < NQS) read_k(ks + 2, kf[(ks + 2) % 3]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) s[kb] = mfma32(kf[ks % 3][kb], qf[ks], s[kb]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    JV_PRIO(0);
+    bf16x8 vf[2][NDB];
+    auto read_v = [&](int sidx, bf16x8 (&f)[NDB]) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) f[db] = *(const bf16x8*)(Vb + vr[sidx] + db * V_DB);
+    };
+    read_v(0, vf[0]);                    // on its way during the softmax
+    __builtin_amdgcn_sched_barrier(0);
+    // interior tile: every key visible to every row of the tile -> no per-element mask
+    const bool interior = (j0 + BN - 1 <= wave_min_pos) && (p.window <= 0 || j0 >= wave_full_begin);
+    float tmax = -INFINITY;
+    if (interior) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) tmax = fmaxf(tmax, s[kb][e]);
+    } else {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int j = j0 + kb * 32 + acc_key(e);
+          const bool ok = row_ok && j <= pos && (p.window <= 0 || j > pos - p.window);
+          const float v = ok ? s[kb][e] : -INFINITY;
+          s[kb][e] = v;
+          tmax = fmaxf(tmax, v);
+        }
+    }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);                          // raw-score units
+    m_run = m_new;
+    // exponents are taken against m_ref, which follows the running maximum only when that has grown
+    // by more than RESCALE_STEP powers of two; most tiles then skip rescaling sums and outputs
+    const bool grown = (m_new - m_ref) * p.scale_log2 > RESCALE_STEP;   // false while no key is visible
+    if (__builtin_amdgcn_ballot_w64(grown) != 0) {
+      const float alpha = grown ? fast_exp2((m_ref - m_new) * p.scale_log2) : 1.f;   // 0 from -inf
+      if (grown) m_ref = m_new;
+      l_lane *= alpha;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[db][e] *= alpha;
+    }
+    const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2;
+    float psum = 0.f;
+    bf16x8 pb[BN / 16];                  // P^T operands: keys 16 s + 8 h .. + 7 = elements 8 (s % 2) .. + 7 of block s / 2
+#pragma unroll
+    for (int sidx = 0; sidx < BN / 16; ++sidx)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pv = fast_exp2(fmaf(s[sidx >> 1][8 * (sidx & 1) + e], p.scale_log2, -m_use));
+        psum += pv;
+        pb[sidx][e] = (bf16_t)pv;
+      }
+    l_lane += psum;
+    JV_PRIO(1);
+#pragma unroll
+    for (int sidx = 0; sidx < BN / 16; ++sidx) {
+      if (sidx + 1 < BN / 16) read_v(sidx + 1, vf[(sidx + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) acc[db] = mfma32(vf[sidx & 1][db], pb[sidx], acc[db]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    JV_PRIO(0);
+  };
+
+  unsigned pg[PCS];
+  if (FAST) {
+    pages_of(j_first, pg);
+    fetch_fast(0, pg);
+    if (next_tile(j_first) < kv_end) pages_of(next_tile(j_first), pg);
+  } else {
+    fetch(j_first, 0);
+  }
+  arrived();
+  if (j_first + BN > kv_end) fix_tail(j_first, 0);
+  __syncthreads();
+  int b = 0;
+  for (int j0 = j_first; j0 < kv_end;) {
+    const int j_next = next_tile(j0);
+    const bool more = j_next < kv_end;
+    if (more) {                                     // in flight while this tile is multiplied; nobody reads that
+      if (FAST) {                                   // buffer: its tile was finished before the last barrier
+        fetch_fast(b ^ 1, pg);
+        const int j_after = next_tile(j_next);
+        if (j_after < kv_end) pages_of(j_after, pg);
+      } else {
+        fetch(j_next, b ^ 1);
+      }
+    }
+    if (wave_live && j0 < wave_kv_end && j0 + BN > wave_kv_begin) multiply(j0, b);
+    arrived();
+    if (more && j_next + BN > kv_end) fix_tail(j_next, b ^ 1);   // own pieces only: no barrier needed before
+    __syncthreads();
+    j0 = j_next;
+    b ^= 1;
+  }
+
+  float l = l_lane + __shfl_xor(l_lane, 32, 64);
+  if (row_ok) {
+    const float inv = 1.f / l;
+    bf16_t* o = p.out + (long long)(q_start + qi) * p.nq * D + (long long)(g * G + hg) * D + h * 4;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {                 // accumulator rows 8i + 4h + j of block db
+        bf16x4 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = (bf16_t)(acc[db][4 * i + j] * inv);
+        *(bf16x4*)(o + db * 32 + i * 8) = v;
+      }
+  }
+}
+#endif
+
 // the host's plan: rows per group, and groups a work item may name
 extern "C" int jv_attn_prefill_group_rows() { return GROUP_ROWS; }
 extern "C" int jv_attn_prefill_groups_per_item() { return RT; }
+// 1: each group of a work item has waves of its own (pair groups that see the same keys); 0: every wave
+// takes rows of both groups (pair a light group with a heavy one)
+#ifdef JV_PREFILL32
+extern "C" int jv_attn_prefill_waves_split() { return 1; }
+#else
+extern "C" int jv_attn_prefill_waves_split() { return 0; }
+#endif
 
 // ------------------------------------------------------------------------------------ decode
 constexpr int BND = 32;  // keys per wave iteration
@@ -765,7 +1182,14 @@ extern "C" int jv_attn_prefill(void* out, const void* q, long long q_row_stride,
   if ((long long)nkv * page_size * D >= (1ll << 31)) return (int)hipErrorInvalidValue;   // offsets inside a page are 32-bit
   if ((long long)n_work * nkv >= (1ll << 31)) return (int)hipErrorInvalidValue;
   const int mode = (a.page_shift >= 3 && a.page_shift <= 6) ? 1 : (a.page_shift > 6 ? 2 : 0);
+#ifdef JV_PREFILL32
+  constexpr bool pow2 = (D & (D - 1)) == 0;
+  void (*kernel)(AttnArgs) = (page_size == 16 && pow2) ? attn_prefill32_kernel<pow2 ? 16 : 1>
+                             : mode == 1 ? attn_prefill32_kernel<1>
+                             : mode == 2 ? attn_prefill32_kernel<2> : attn_prefill32_kernel<0>;
+#else
   void (*kernel)(AttnArgs) = mode == 1 ? attn_prefill_kernel<1> : (mode == 2 ? attn_prefill_kernel<2> : attn_prefill_kernel<0>);
+#endif
   hipLaunchKernelGGL(kernel, dim3(n_work * nkv), dim3(256), 0, (hipStream_t)stream, a);
   return JV_LAUNCH_CHECK();
 }

@@ -530,8 +530,16 @@ MFMA_ATTENTION_MAX_HEAD_DIM = 256
 
 def attn_prefill_geometry(head_dim: int) -> tuple[int, int]:
     """(rows of a group, groups a work item of the prefill kernel may name).  A row is a (query,
-    head-in-group) pair; a block's 4 waves take 16 rows each of every group of its item."""
+    head-in-group) pair."""
     return 64, (2 if head_dim <= 128 else 1)
+
+
+def attn_prefill_waves_split(head_dim: int) -> bool:
+    """Whether each group of a work item has waves of its own (head sizes 32, 64, 96, 128: two waves
+    of 32 rows per group), so that a block is busy only while both groups see keys: neighbouring
+    groups belong together.  Otherwise each of the 4 waves takes 16 rows of every group, and pairing
+    a light group with a heavy one evens out the blocks."""
+    return head_dim % 32 == 0 and head_dim <= 128
 
 
 _checked_attention_libraries = set()
@@ -544,8 +552,9 @@ def _attention_library(head_dim: int):
     if head_dim not in _checked_attention_libraries:
         lib.jv_attn_decode_scratch_floats.restype = c_longlong
         got = (lib.jv_attn_head_dim(), lib.jv_attn_prefill_group_rows(), lib.jv_attn_prefill_groups_per_item(),
-               lib.jv_attn_decode_scratch_floats(c_int(3), c_int(5), c_int(7)))
-        want = (head_dim, *attn_prefill_geometry(head_dim), attn_decode_scratch_floats(3, 5, 7, head_dim))
+               bool(lib.jv_attn_prefill_waves_split()), lib.jv_attn_decode_scratch_floats(c_int(3), c_int(5), c_int(7)))
+        want = (head_dim, *attn_prefill_geometry(head_dim), attn_prefill_waves_split(head_dim),
+                attn_decode_scratch_floats(3, 5, 7, head_dim))
         if got != want:
             raise KernelArgumentError(f"attention library for head size {head_dim} reports {got}, the planner expects {want}")
         _checked_attention_libraries.add(head_dim)

@@ -3,8 +3,10 @@
 bfloat16 with a head size and page size the matrix-core kernels are built for: requests with
 one token in the step go to the decode kernel (keys shared out to several blocks when few
 requests would leave the chip idle), all others to the prefill kernel in groups of 64 (query,
-head-in-group) rows; a work item pairs a group that sees many keys with one of the same request
-that sees few, so that all blocks carry the same load, heaviest items first.  Everything else
+head-in-group) rows; a work item names two groups of one request, heaviest items first: two
+neighbours where the kernel gives each group waves of its own (they see the same keys), else,
+while all blocks are on the chip at once, a group that sees many keys with one that sees few, so
+that all blocks carry the same load.  Everything else
 (float32, other head sizes) runs the generic float-math kernel.  The plan depends on the
 step's lengths, the heads-per-group ratio and whether the layer has a window, so it is built
 once per step and shared by all layers alike.
@@ -79,16 +81,22 @@ def prefill_work_items(q_lens, context_lens, g: int, window: int, group_rows: in
     return [(r, a, b) for _, r, a, b in items]
 
 
-def prefill_item_shape(rows: int, nkv: int, group_rows: int, kernel_groups: int, compute_units: int):
+def prefill_item_shape(rows: int, nkv: int, group_rows: int, kernel_groups: int, compute_units: int,
+                       waves_split: bool = False):
     """(groups per work item, whether light groups are paired with heavy ones) for a step with
-    ``rows`` (query, head-in-group) rows per kv head in its prompt portions.  Measured on 32 q heads,
-    8 kv heads of 128: while items of two groups would not even give every compute unit a block,
+    ``rows`` (query, head-in-group) rows per kv head in its prompt portions.  A kernel whose groups
+    have waves of their own (``waves_split``) always gets neighbouring pairs: half of a block's waves
+    would idle through the keys that only one group sees (2,048 tokens, 32 q heads over 8 kv heads
+    of 128: 64 against 78 us; one group per item: 88).  For the other kernel, measured on the same
+    heads: while items of two groups would not even give every compute unit a block,
     items of one group do better although every block then loads its keys for half the rows
     (512 tokens after 3,000: 111 against 135 us; after 16,000: 507 against 622); balancing wins
     while all blocks are on the chip at once, two per compute unit (2,048 tokens, 512 blocks: 88
     against 98 us); one more block and the equal loads need a whole further round, so neighbours
     that share their keys, heaviest first, win from there (2,304 tokens, 576 blocks: 111 against
     137 us; 8,192: 887 against 1,036)."""
+    if waves_split:
+        return kernel_groups, False
     blocks = -(-rows // (group_rows * kernel_groups)) * nkv
     if kernel_groups > 1 and blocks <= compute_units:
         return 1, True
@@ -99,7 +107,8 @@ def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> Mfm
     g = nq // nkv
     group_rows, kernel_groups = K.attn_prefill_geometry(head_dim)
     rows = sum(ql * g for ql in ctx.q_lens_host if ql > 1)
-    groups_per_item, balance = prefill_item_shape(rows, nkv, group_rows, kernel_groups, K.compute_units(device))
+    groups_per_item, balance = prefill_item_shape(rows, nkv, group_rows, kernel_groups, K.compute_units(device),
+                                                  K.attn_prefill_waves_split(head_dim))
     prefill = prefill_work_items(ctx.q_lens_host, ctx.context_lens_host, g, window, group_rows, groups_per_item,
                                  balance=balance)
     decode = [r for r, ql in enumerate(ctx.q_lens_host) if ql == 1]

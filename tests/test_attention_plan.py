@@ -62,6 +62,9 @@ def test_item_shape_follows_the_fill_of_the_chip():
     assert shape(2048) == (2, True)                                      # 512 blocks: all on the chip at once
     assert shape(2304) == (2, False) and shape(8192) == (2, False)       # one more round of blocks
     assert prefill_item_shape(100, 8, 64, 1, 256) == (1, True)           # a kernel with one group per item stays so
+    # a kernel whose groups have waves of their own always gets two neighbouring groups
+    split = lambda tokens: prefill_item_shape(tokens * 4, 8, 64, 2, 256, waves_split=True)
+    assert split(64) == split(512) == split(2048) == split(8192) == (2, False)
     # every row still lands in exactly one item
     items = prefill_work_items([600], [37], 4, 0, 64, 1)
     rows = sorted(m0 for _, m0, other in items if other == -1)

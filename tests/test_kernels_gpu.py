@@ -477,18 +477,28 @@ MFMA_PREFILL_CASES = [c for c in ATT_CASES if c[3] % 8 == 0] + [
     (4, 1, 128, 32, [(64, 129), (0, 64)], 40),
     (2, 1, 16, 8, [(17000, 40)], None),    # more pages than the kernel keeps of the table at a time
     (2, 1, 16, 8, [(17000, 200)], 100),
+    # head sizes of the kernel with 32-row tiles, in each of its ways of finding a key's page
+    (6, 2, 96, 16, [(70, 90), (0, 5)], None),       # keys of 12 chunks: a load instruction spans pages
+    (4, 2, 128, 24, [(100, 140)], None),            # a page size that is no power of two
+    (4, 1, 64, 128, [(200, 100), (0, 129)], None),  # pages larger than a key tile
+    (4, 2, 128, 8, [(3, 150)], 90),
+    (6, 3, 32, 16, [(1, 260), (500, 33)], None),    # one load instruction a tile and wave
+    (2, 1, 32, 8, [(9000, 70)], None),              # more pages than the general path keeps of the table at a time
+    (10, 2, 64, 16, [(64, 64), (63, 65), (0, 2)], None),   # 5 heads a group: a query's rows cross the 32-row tiles
+    (32, 8, 128, 16, [(1900, 300)], 1024),          # window wider than the portion: early tiles drop out one by one
 ]
 
 
 def _prefill_work(reqs, g, d, window, plan):
-    """Work items of the prefill kernel: by the engine's planner, one group per item, or every group
-    in the item's second place."""
+    """Work items of the prefill kernel: by the engine's planner (in both its ways of pairing groups),
+    one group per item, every group in the item's second place, or the first group with the last."""
     from jax_vllm_amd.parts.attention_backend import prefill_work_items
 
     group_rows, per_item = K().attn_prefill_geometry(d)
     singles = [(r, m0) for r, (c, ql) in enumerate(reqs) for m0 in range(0, ql * g, group_rows)]
-    if plan == "planner":
-        items = prefill_work_items([ql for _, ql in reqs], [c for c, _ in reqs], g, window or 0, group_rows, per_item)
+    if plan in ("planner", "neighbours"):       # light groups paired with heavy ones, or neighbours paired
+        items = prefill_work_items([ql for _, ql in reqs], [c for c, _ in reqs], g, window or 0, group_rows, per_item,
+                                   balance=plan == "planner")
         items += [(r, 0, -1) for r, (c, ql) in enumerate(reqs) if ql == 1]      # the planner leaves these to decode
     elif plan == "second" and per_item > 1:
         items = [(r, -1, m0) for r, m0 in singles]
@@ -506,7 +516,7 @@ def _prefill_work(reqs, g, d, window, plan):
     return torch.tensor([x for it in items for x in it], dtype=torch.int32).cuda(), len(items)
 
 
-@pytest.mark.parametrize("plan", ["planner", "single", "second", "far"])
+@pytest.mark.parametrize("plan", ["planner", "neighbours", "single", "second", "far"])
 @pytest.mark.parametrize("case", MFMA_PREFILL_CASES,
                          ids=[f"h{c[0]}g{c[1]}d{c[2]}p{c[3]}w{c[5]}n{len(c[4])}" for c in MFMA_PREFILL_CASES])
 def test_mfma_prefill_attention(case, plan):
