@@ -88,57 +88,59 @@ __device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
 
 #define ARN_MAX_V 8
 #define ARN_MAX_PARTS 4
-template <typename T>
-__global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
-                                       const float* __restrict__ w, T* __restrict__ out,
-                                       const int* __restrict__ rows, int hidden, float eps) {
+// V = 16-byte pieces of the residual row per thread (the launch picks the least that covers the row).  Every
+// load (residual, delta, norm weight) is issued before the reduction and none sits inside a branch: a
+// piece beyond the row reads the row's last piece again and only its stores and its share of the sum are
+// left out (a load inside a branch makes the compiler wait for all loads in flight where the branch
+// ends: 1.1 us of a 4.4 us kernel).  A short row's time is the sum of its dependent memory round trips.
+template <typename T, int V>
+__global__ void __launch_bounds__(256)
+add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
+                       const float* __restrict__ w, T* __restrict__ out,
+                       const int* __restrict__ rows, int hidden, float eps) {
   __shared__ float red[32];
   const long long i = blockIdx.x;
   const long long r = rows ? (long long)rows[i] : i;
   float* hr = h + r * hidden;
-  const T* dr = delta ? delta + r * hidden : nullptr;
+  const T* dr = delta ? delta + r * hidden : (const T*)w;      // any readable address: its values get no weight
   T* o = out + i * hidden;
   const int nvec = hidden >> 2;
-  // every load (residual, delta, norm weight) is issued before the reduction: a short row's time is
-  // the sum of its dependent memory round trips, and the weights are cold in every layer
-  float4 x[ARN_MAX_V], ww[ARN_MAX_V];
+  float4 x[V], ww[V], d[V];
+#pragma unroll
+  for (int k = 0; k < V; ++k) {
+    const int c = min((int)(threadIdx.x + k * blockDim.x), nvec - 1);
+    ww[k] = *(const float4*)(w + 4 * c);
+    x[k] = *(const float4*)(hr + 4 * c);
+    d[k] = load4<T>(dr + (delta ? 4 * c : 0));
+  }
   float ss = 0.f;
 #pragma unroll
-  for (int k = 0; k < ARN_MAX_V; ++k) {
+  for (int k = 0; k < V; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
-    if (c < nvec) ww[k] = *(const float4*)(w + 4 * c);
-  }
-#pragma unroll
-  for (int k = 0; k < ARN_MAX_V; ++k) {
-    const int c = threadIdx.x + k * blockDim.x;
+    float4 v = x[k];
+    if (delta) { v.x += d[k].x; v.y += d[k].y; v.z += d[k].z; v.w += d[k].w; }
     if (c < nvec) {
-      float4 v = *(const float4*)(hr + 4 * c);
-      if (dr) {
-        const float4 d = load4<T>(dr + 4 * c);
-        v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
-        if (!rows) *(float4*)(hr + 4 * c) = v;
-      }
-      x[k] = v;
+      if (delta && !rows) *(float4*)(hr + 4 * c) = v;
       ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
+    x[k] = v;
   }
   ss = block_sum(ss, red);
   const float inv = rsqrtf(ss / (float)hidden + eps);
 #pragma unroll
-  for (int k = 0; k < ARN_MAX_V; ++k) {
+  for (int k = 0; k < V; ++k) {
     const int c = threadIdx.x + k * blockDim.x;
-    if (c < nvec) {
-      const float4 v = x[k];
+    const float4 v = x[k];
+    if (c < nvec)
       store4<T>(o + 4 * c, float4{v.x * inv * ww[k].x, v.y * inv * ww[k].y, v.z * inv * ww[k].z, v.w * inv * ww[k].w});
-    }
   }
 }
 
 // The same with the delta given as NP float partial products of a matrix product whose inner
 // size was shared out to NP blocks: parts[q][r][:], added first, in the order of q, then to the
-// residual.  Every load of the row is issued before anything is computed (the kernel's time is
-// its chain of memory round trips).
-template <typename T, int NP>
+// residual.
+// EXACT: blocks of 256 threads whose V pieces cover the row exactly (no index is clamped or tested).
+template <typename T, int NP, int V, bool EXACT>
 __global__ void __launch_bounds__(256)
 add_rmsnorm_parts_kernel(float* __restrict__ h, const float* __restrict__ parts, long long part_stride,
                          const float* __restrict__ w, T* __restrict__ out, const int* __restrict__ rows,
@@ -149,43 +151,80 @@ add_rmsnorm_parts_kernel(float* __restrict__ h, const float* __restrict__ parts,
   float* hr = h + r * hidden;
   const float* pr = parts + r * hidden;
   T* o = out + i * hidden;
-  const int nvec = hidden >> 2;
-  float4 x[ARN_MAX_V], ww[ARN_MAX_V], e[ARN_MAX_V][NP];
+  const int nvec = EXACT ? V * 256 : hidden >> 2;
+  const int nthreads = EXACT ? 256 : blockDim.x;
+  float4 x[V], ww[V], e[V][NP];
 #pragma unroll
-  for (int k = 0; k < ARN_MAX_V; ++k) {
-    const int c = threadIdx.x + k * blockDim.x;
-    if (c < nvec) {
-      ww[k] = *(const float4*)(w + 4 * c);
-      x[k] = *(const float4*)(hr + 4 * c);
+  for (int k = 0; k < V; ++k) {
+    const int c = EXACT ? (int)threadIdx.x + k * 256 : min((int)(threadIdx.x + k * nthreads), nvec - 1);
+    ww[k] = *(const float4*)(w + 4 * c);
+    x[k] = *(const float4*)(hr + 4 * c);
 #pragma unroll
-      for (int q = 0; q < NP; ++q) e[k][q] = *(const float4*)(pr + q * part_stride + 4 * c);
-    }
+    for (int q = 0; q < NP; ++q) e[k][q] = *(const float4*)(pr + q * part_stride + 4 * c);
   }
   float ss = 0.f;
 #pragma unroll
-  for (int k = 0; k < ARN_MAX_V; ++k) {
-    const int c = threadIdx.x + k * blockDim.x;
-    if (c < nvec) {
-      float4 d = e[k][0];
+  for (int k = 0; k < V; ++k) {
+    const int c = threadIdx.x + k * nthreads;
+    float4 d = e[k][0];
 #pragma unroll
-      for (int q = 1; q < NP; ++q) { d.x += e[k][q].x; d.y += e[k][q].y; d.z += e[k][q].z; d.w += e[k][q].w; }
-      float4 v = x[k];
-      v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+    for (int q = 1; q < NP; ++q) { d.x += e[k][q].x; d.y += e[k][q].y; d.z += e[k][q].z; d.w += e[k][q].w; }
+    float4 v = x[k];
+    v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+    if (EXACT || c < nvec) {
       if (!rows) *(float4*)(hr + 4 * c) = v;
-      x[k] = v;
       ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
     }
+    x[k] = v;
   }
   ss = block_sum(ss, red);
   const float inv = rsqrtf(ss / (float)hidden + eps);
 #pragma unroll
-  for (int k = 0; k < ARN_MAX_V; ++k) {
-    const int c = threadIdx.x + k * blockDim.x;
-    if (c < nvec) {
-      const float4 v = x[k];
+  for (int k = 0; k < V; ++k) {
+    const int c = threadIdx.x + k * nthreads;
+    const float4 v = x[k];
+    if (EXACT || c < nvec)
       store4<T>(o + 4 * c, float4{v.x * inv * ww[k].x, v.y * inv * ww[k].y, v.z * inv * ww[k].z, v.w * inv * ww[k].w});
-    }
   }
+}
+
+// threads of a block and 16-byte pieces per thread for a row of nvec pieces (nvec <= 8 * 256)
+static void arn_shape(int nvec, int* threads, int* v) {
+  *threads = nvec >= 1024 ? 256 : (nvec >= 256 ? 128 : 64);
+  const int need = (nvec + *threads - 1) / *threads;
+  *v = need <= 1 ? 1 : need <= 2 ? 2 : need <= 4 ? 4 : need <= 5 ? 5 : 8;
+}
+template <typename T>
+static void launch_arn_vec(int v, int n_out, int threads, hipStream_t st, float* h, const T* delta, const float* w, T* out,
+                           const int* rows, int hidden, float eps) {
+#define ARN_GO(V) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<T, V>), dim3(n_out), dim3(threads), 0, st, h, delta, w, out, rows, hidden, eps)
+  switch (v) {
+    case 1: ARN_GO(1); break;
+    case 2: ARN_GO(2); break;
+    case 4: ARN_GO(4); break;
+    case 5: ARN_GO(5); break;
+    default: ARN_GO(8); break;
+  }
+#undef ARN_GO
+}
+template <typename T, int NP>
+static void launch_arn_parts(int v, int n_out, int threads, hipStream_t st, float* h, const float* parts, long long part_stride,
+                             const float* w, T* out, const int* rows, int hidden, float eps) {
+#define ARN_GO(V)                                                                                                \
+  if (threads == 256 && hidden == 4 * 256 * V)                                                                   \
+    hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, NP, V, true>), dim3(n_out), dim3(256), 0, st, h, parts,       \
+                       part_stride, w, out, rows, hidden, eps);                                                  \
+  else                                                                                                           \
+    hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, NP, V, false>), dim3(n_out), dim3(threads), 0, st, h, parts,  \
+                       part_stride, w, out, rows, hidden, eps)
+  switch (v) {
+    case 1: ARN_GO(1); break;
+    case 2: ARN_GO(2); break;
+    case 4: ARN_GO(4); break;
+    case 5: ARN_GO(5); break;
+    default: ARN_GO(8); break;
+  }
+#undef ARN_GO
 }
 
 // ---------------------------------------------------------------- plain RMSNorm over the last axis
@@ -275,10 +314,10 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
     if (n_out <= 0) return 0;                                                                       \
     const int threads = hidden >= 2048 ? 512 : 256;                                                 \
     if (hidden % 4 == 0 && hidden <= 4 * ARN_MAX_V * 256) {                                         \
-      const int nvec = hidden / 4;                                                                  \
-      const int vt = nvec >= 1024 ? 256 : (nvec >= 256 ? 128 : 64);                                 \
-      hipLaunchKernelGGL(add_rmsnorm_vec_kernel<T>, dim3(n_out), dim3(vt), 0, (hipStream_t)stream,  \
-                         h, (const T*)delta, w, (T*)out, rows, hidden, eps);                        \
+      int vt, v;                                                                                    \
+      arn_shape(hidden / 4, &vt, &v);                                                               \
+      launch_arn_vec<T>(v, n_out, vt, (hipStream_t)stream, h, (const T*)delta, w, (T*)out, rows,    \
+                        hidden, eps);                                                               \
     } else {                                                                                        \
       hipLaunchKernelGGL(add_rmsnorm_kernel<T>, dim3(n_out), dim3(threads), 0, (hipStream_t)stream, \
                          h, (const T*)delta, w, (T*)out, rows, hidden, eps);                        \
@@ -293,18 +332,14 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
     if (n_out <= 0) return 0;                                                                       \
     if (n_parts < 1 || n_parts > ARN_MAX_PARTS || hidden % 4 != 0 || hidden > 4 * ARN_MAX_V * 256)  \
       return (int)hipErrorInvalidValue;                                                             \
-    const int nvec = hidden / 4;                                                                    \
-    const int vt = nvec >= 1024 ? 256 : (nvec >= 256 ? 128 : 64);                                   \
+    int vt, v;                                                                                      \
+    arn_shape(hidden / 4, &vt, &v);                                                                 \
     hipStream_t st = (hipStream_t)stream;                                                           \
     switch (n_parts) {                                                                              \
-      case 1: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 1>), dim3(n_out), dim3(vt), 0, st, h, \
-                                 parts, part_stride, w, (T*)out, rows, hidden, eps); break;         \
-      case 2: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 2>), dim3(n_out), dim3(vt), 0, st, h, \
-                                 parts, part_stride, w, (T*)out, rows, hidden, eps); break;         \
-      case 3: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 3>), dim3(n_out), dim3(vt), 0, st, h, \
-                                 parts, part_stride, w, (T*)out, rows, hidden, eps); break;         \
-      default: hipLaunchKernelGGL((add_rmsnorm_parts_kernel<T, 4>), dim3(n_out), dim3(vt), 0, st,   \
-                                  h, parts, part_stride, w, (T*)out, rows, hidden, eps); break;     \
+      case 1: launch_arn_parts<T, 1>(v, n_out, vt, st, h, parts, part_stride, w, (T*)out, rows, hidden, eps); break; \
+      case 2: launch_arn_parts<T, 2>(v, n_out, vt, st, h, parts, part_stride, w, (T*)out, rows, hidden, eps); break; \
+      case 3: launch_arn_parts<T, 3>(v, n_out, vt, st, h, parts, part_stride, w, (T*)out, rows, hidden, eps); break; \
+      default: launch_arn_parts<T, 4>(v, n_out, vt, st, h, parts, part_stride, w, (T*)out, rows, hidden, eps); break; \
     }                                                                                               \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \

@@ -106,6 +106,9 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_kernel(
 // multiple of 64 (D = 128 or 256 fully rotated): lane l holds elements l, l+64, ..., so both
 // members of every rotation pair sit in one lane: no LDS, no barrier.  One wave takes
 // `heads_per_wave` consecutive heads of one token.
+// No load sits inside a branch (one that does makes the compiler wait, where the branch ends, for
+// every load in flight, and a step of few tokens is a chain of memory round trips): what is not
+// there (no rotation, no norm weight, no slot) is read from the row itself and given no weight.
 template <typename T, int E, int NP>
 __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
     T* __restrict__ qkv, const float* __restrict__ parts, long long part_stride,
@@ -118,24 +121,37 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
   const long long t = blockIdx.x;
   const int n_heads = nq + 2 * nkv;
   T* row = qkv + t * (long long)n_heads * D;
-  const long long slot = slot_mapping ? (long long)slot_mapping[t] : -1;
-  const bool store = (slot >= 0) && (k_pages != nullptr);
-  const long long page = store ? slot / page_size : 0;
-  const int off = store ? (int)(slot - page * page_size) : 0;
   const int half = rotary_dim / 2, HE = half / 64;   // pair (e, e + HE) for e < HE
-  float cs[E], sn[E];                                 // cos/sin of this lane's pair indices
-  if (cos_sin) {
-#pragma unroll
-    for (int e = 0; e < E; ++e)
-      if (e < HE) {
-        cs[e] = cos_sin[t * rotary_dim + e * 64 + lane];
-        sn[e] = cos_sin[t * rotary_dim + half + e * 64 + lane];
-      }
-  }
   const int h0 = (blockIdx.y * 4 + wid) * heads_per_wave;
+  if (h0 >= walk_heads) return;                       // the whole wave
+  // everything that does not depend on the head: slot, cos/sin of this lane's pair indices
+  // the slot through the vector unit (an index the compiler cannot see through): a scalar load would be
+  // waited for before the loads below are even asked for
+  int lane_zero;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
+  const int* slot_at = slot_mapping ? slot_mapping + t : (const int*)row;
+  const int slot_raw = slot_at[lane_zero];
+  float cs[E], sn[E];
+  {
+    // without a table: the row itself, read as floats (at least 3 heads of D elements of 2 bytes: long enough)
+    const float* cp = cos_sin ? cos_sin + t * rotary_dim + lane : (const float*)row + lane;
+    const int hh = cos_sin ? half : 0;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const int ee = e < HE ? e : 0;
+      cs[e] = cp[ee * 64];
+      sn[e] = cp[hh + ee * 64];
+    }
+  }
   for (int head = h0; head < h0 + heads_per_wave && head < walk_heads; ++head) {
     T* x = row + (long long)head * D;
     float v[E], wv[E];
+    {  // the norm weights are asked for together with the head, not after its reduction
+      const float* w0 = head < nq ? q_w : (head < nq + nkv ? k_w : nullptr);
+      const float* wp = (w0 ? w0 : (const float*)row) + lane;
+#pragma unroll
+      for (int e = 0; e < E; ++e) wv[e] = wp[e * 64];      // used only where there is a weight
+    }
     if (NP == 0) {
 #pragma unroll
       for (int e = 0; e < E; ++e) v[e] = to_f32(x[e * 64 + lane]);
@@ -155,11 +171,11 @@ __global__ void __launch_bounds__(256) qk_norm_rope_write_fast_kernel(
         for (int q = 1; q < NP; ++q) v[e] += pv[q][e];
       }
     }
-    {  // the norm weights are asked for together with the head, not after its reduction
-      const float* w0 = head < nq ? q_w : (head < nq + nkv ? k_w : nullptr);
-#pragma unroll
-      for (int e = 0; e < E; ++e) wv[e] = w0 ? w0[e * 64 + lane] : 1.f;
-    }
+    // the slot is looked at only here, after every load of the head has been asked for
+    const long long slot = slot_mapping ? (long long)__builtin_amdgcn_readfirstlane(slot_raw) : -1;
+    const bool store = (slot >= 0) && (k_pages != nullptr);
+    const long long page = store ? slot / page_size : 0;
+    const int off = store ? (int)(slot - page * page_size) : 0;
     if (head >= nq + nkv) {  // v head: copied to its (transposed) page
       if (store) {
         T* dst = v_pages + (page * nkv + (head - nq - nkv)) * (long long)D * page_size + off;
