@@ -508,7 +508,12 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
 //   * both tiles are stored in 16-byte chunks whose position inside each 256-byte line is
 //     xor-ed with the line number: reads of 32 rows at one column and writes of whole rows are
 //     both conflict-free (measured).
-// Tiles are double-buffered in LDS: one barrier per 64 keys.
+// Tiles are double-buffered in LDS: one barrier per 64 keys.  With pages of 16 keys and a head size
+// that is a power of two (PIPE) a wave also overlaps its own work: the scores of tile i + 1 are
+// multiplied while the probabilities of tile i are made (measured at 32 q heads over 8 kv heads of
+// 128: 2,048 tokens 58 against 63 us, 8,192 tokens 566 against 638, 512 tokens after 16,000: 306
+// against 383; the kernel then keeps the matrix unit busy 55..60 % of the time at the 1.9 GHz it
+// runs at, the LDS about as much, and neither can be filled further by two waves a SIMD).
 #ifdef JV_PREFILL32
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 // a wave in a burst of products goes first: the other wave of its SIMD (of the compute unit's other block) then
@@ -525,7 +530,7 @@ constexpr int PCS = BN * CPK / 256;        // 16-byte pieces of a K tile (and of
 constexpr bool KB_ADDS = (32 * CPK / 16) % 16 == 0;   // the second key block's chunks are the first's plus a constant
 __device__ __forceinline__ int swizzle(int q) { return q ^ ((q >> 4) & 15); }   // chunk index -> chunk position
 
-template <int PAGES>
+template <int PAGES, bool PIPE = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) attn_prefill32_kernel(AttnArgs p) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[2][BN * D];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[2][D * BN];
@@ -646,8 +651,17 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       v_off[i] = (g * D + d) * P + (PAGES == 1 ? ((kc * 8) & (P - 1)) : 0);
     }
   }
-  typedef const __attribute__((address_space(1))) void* gptr_t;
-  typedef __attribute__((address_space(3))) void* lptr_t;
+  // 16 bytes a lane from global memory straight into LDS: lane l of the wave writes to `lds` + 16 l.  Written
+  // in assembly on purpose: told that a vector-memory instruction writes LDS, the compiler waits for ALL
+  // such loads in flight before every LDS read it cannot prove to be elsewhere (it cannot tell the two
+  // buffers apart), which is exactly the overlap this kernel is built on.  The waits are ours: arrived()
+  // before the barrier that hands a buffer over.
+  typedef const bf16_t* gptr_t;
+  typedef const bf16_t* lptr_t;
+  auto dma16 = [&](gptr_t src, lptr_t lds) {
+    const unsigned at = (unsigned)(unsigned long long)(const __attribute__((address_space(3))) void*)lds;
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(at) : "memory", "m0");
+  };
   // Nothing here looks at a loaded value.  A piece past the last key reads the same slot of the last
   // page (allocated memory): K there is masked by position, V is zeroed in LDS by fix_tail.
   // fast path: the PCS pages of this wave's instructions for the tile at j0, as scalars from the
@@ -667,10 +681,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
     for (int i = 0; i < PCS; ++i) {
       const unsigned long long base = (unsigned long long)pg[i] * page_stride;   // scalar
-      __builtin_amdgcn_global_load_lds((gptr_t)(p.k_pages + base + (unsigned)k_off[i]),
-                                       (lptr_t)&Ks[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((gptr_t)(p.v_pages + base + (unsigned)v_off[i]),
-                                       (lptr_t)&Vs[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
+      dma16(p.k_pages + base + (unsigned)k_off[i],
+              &Ks[b][(4 * i + wave) * 64 * 8]);
+      dma16(p.v_pages + base + (unsigned)v_off[i],
+              &Vs[b][(4 * i + wave) * 64 * 8]);
     }
   };
   auto fetch = [&](int j0, int b) {
@@ -694,8 +708,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       }
       if (pi > end_page) pi = end_page;
       const unsigned page = (unsigned)page_ids[pi];
-      __builtin_amdgcn_global_load_lds((gptr_t)(p.k_pages + ((unsigned long long)page * page_stride + (unsigned)off)),
-                                       (lptr_t)&Ks[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
+      dma16(p.k_pages + ((unsigned long long)page * page_stride + (unsigned)off),
+              &Ks[b][(4 * i + wave) * 64 * 8]);
     }
 #pragma unroll
     for (int i = 0; i < PCS; ++i) {
@@ -709,8 +723,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       }
       if (pi > end_page) pi = end_page;
       const unsigned page = (unsigned)page_ids[pi];
-      __builtin_amdgcn_global_load_lds((gptr_t)(p.v_pages + ((unsigned long long)page * page_stride + (unsigned)off)),
-                                       (lptr_t)&Vs[b][(4 * i + wave) * 64 * 8], 16, 0, 0);
+      dma16(p.v_pages + ((unsigned long long)page * page_stride + (unsigned)off),
+              &Vs[b][(4 * i + wave) * 64 * 8]);
     }
   };
   // V entries of keys at or past kv_end become zeros (their probabilities are zeros, and zero times a
@@ -845,6 +859,219 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     JV_PRIO(0);
   };
 
+  if constexpr (PIPE && FAST) {
+    // ---- the same walk with a wave's products and its softmax overlapped: while the probabilities of tile i
+    // are made (float units), the scores of tile i + 1 are already multiplied (matrix unit), and the first
+    // products of O^T += V^T P^T start as soon as their 16 keys' probabilities exist.  K is therefore
+    // fetched two tiles ahead and V one: K(i+2) goes where K(i) was, V(i+1) where V(i-1) was.
+    auto fetch_k = [&](int b, const unsigned (&pgs)[PCS]) {
+#pragma unroll
+      for (int i = 0; i < PCS; ++i)
+        dma16(p.k_pages + (unsigned long long)pgs[i] * page_stride + (unsigned)k_off[i],
+              &Ks[b][(4 * i + wave) * 64 * 8]);
+    };
+    auto fetch_v = [&](int b, const unsigned (&pgs)[PCS]) {
+#pragma unroll
+      for (int i = 0; i < PCS; ++i)
+        dma16(p.v_pages + (unsigned long long)pgs[i] * page_stride + (unsigned)v_off[i],
+              &Vs[b][(4 * i + wave) * 64 * 8]);
+    };
+    auto read_k = [&](const bf16_t* Kb, int ks, bf16x8 (&f)[2]) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) f[kb] = *(const bf16x8*)(Kb + (KB_ADDS ? kr[ks] + kb * 32 * D : k_read(kb, ks)));
+    };
+    auto read_v = [&](const bf16_t* Vb, int sidx, bf16x8 (&f)[NDB]) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) f[db] = *(const bf16x8*)(Vb + vr[sidx] + db * V_DB);
+    };
+    auto qk_step = [&](f32x16 (&sn)[2], const bf16x8 (&f)[2], int ks) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) sn[kb] = mfma32(f[kb], qf[ks], sn[kb]);
+    };
+    auto pv_step = [&](const bf16x8 (&f)[NDB], const bf16x8& pbs) {
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) acc[db] = mfma32(f[db], pbs, acc[db]);
+    };
+    // the row's maximum over the tile, the new reference if it has grown; returns whether any row of the wave moved
+    auto row_max = [&](f32x16 (&sc)[2], int j0, float& alpha) -> bool {
+      const bool interior = (j0 + BN - 1 <= wave_min_pos) && (p.window <= 0 || j0 >= wave_full_begin);
+      float tmax = -INFINITY;
+      if (interior) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) tmax = fmaxf(tmax, sc[kb][e]);
+      } else {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int j = j0 + kb * 32 + acc_key(e);
+            const bool ok = row_ok && j <= pos && (p.window <= 0 || j > pos - p.window);
+            const float v = ok ? sc[kb][e] : -INFINITY;
+            sc[kb][e] = v;
+            tmax = fmaxf(tmax, v);
+          }
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run, tmax);
+      m_run = m_new;
+      const bool grown = (m_new - m_ref) * p.scale_log2 > RESCALE_STEP;
+      alpha = grown ? fast_exp2((m_ref - m_new) * p.scale_log2) : 1.f;
+      if (grown) m_ref = m_new;
+      return __builtin_amdgcn_ballot_w64(grown) != 0;
+    };
+    auto rescale = [&](float alpha) {
+      l_lane *= alpha;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[db][e] *= alpha;
+    };
+    auto exp_chunk = [&](const f32x16 (&sc)[2], int sidx, float m_use, bf16x8& pbs) {
+      float psum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float pv = fast_exp2(fmaf(sc[sidx >> 1][8 * (sidx & 1) + e], p.scale_log2, -m_use));
+        psum += pv;
+        pbs[e] = (bf16_t)pv;
+      }
+      l_lane += psum;
+    };
+    constexpr int NPS = BN / 16;                       // products O^T += V^T P^T of 16 keys each
+    // scores of the next tile only (the wave sees nothing of this one)
+    auto tile_qk = [&](f32x16 (&sn)[2], const bf16_t* Kb) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sn[kb][e] = 0.f;
+      bf16x8 kf[2][2];
+      read_k(Kb, 0, kf[0]);
+#pragma unroll
+      for (int ks = 0; ks < NQS; ++ks) {
+        if (ks + 1 < NQS) read_k(Kb, ks + 1, kf[(ks + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        qk_step(sn, kf[ks & 1], ks);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // softmax and output products of this tile only
+    auto tile_sm = [&](f32x16 (&sc)[2], int j0, const bf16_t* Vb) {
+      bf16x8 vf[2][NDB], pb[NPS];
+      read_v(Vb, 0, vf[0]);
+      float alpha;
+      if (row_max(sc, j0, alpha)) rescale(alpha);
+      const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2;
+#pragma unroll
+      for (int sidx = 0; sidx < NPS; ++sidx) exp_chunk(sc, sidx, m_use, pb[sidx]);
+#pragma unroll
+      for (int sidx = 0; sidx < NPS; ++sidx) {
+        if (sidx + 1 < NPS) read_v(Vb, sidx + 1, vf[(sidx + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        pv_step(vf[sidx & 1], pb[sidx]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    // both: scores of the next tile under the softmax of this one
+    auto tile_both = [&](f32x16 (&sc)[2], f32x16 (&sn)[2], int j0, const bf16_t* Kb, const bf16_t* Vb) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sn[kb][e] = 0.f;
+      constexpr int SPG = (NQS + 3) / 4;               // score steps per group (4 groups, one per 16 keys of probabilities)
+      bf16x8 kf[2][SPG][2], vf[2][NDB], pb[NPS];
+      auto read_group = [&](int gidx, bf16x8 (&f)[SPG][2]) {
+#pragma unroll
+        for (int i = 0; i < SPG; ++i)
+          if (gidx * SPG + i < NQS) read_k(Kb, gidx * SPG + i, f[i]);
+      };
+      auto qk_group = [&](int gidx, const bf16x8 (&f)[SPG][2]) {
+#pragma unroll
+        for (int i = 0; i < SPG; ++i)
+          if (gidx * SPG + i < NQS) qk_step(sn, f[i], gidx * SPG + i);
+      };
+      read_group(0, kf[0]);
+      // group 0: first score steps under the row maximum
+      read_group(1, kf[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      JV_PRIO(1);
+      qk_group(0, kf[0]);
+      float alpha;
+      const bool moved = row_max(sc, j0, alpha);
+      __builtin_amdgcn_sched_barrier(0);
+      if (moved) rescale(alpha);
+      const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref * p.scale_log2;
+      // groups 1..3: score steps under the exponentials of keys 0..47
+#pragma unroll
+      for (int gidx = 1; gidx < 4; ++gidx) {
+        if (gidx + 1 < 4) read_group(gidx + 1, kf[(gidx + 1) & 1]);
+        else read_v(Vb, 0, vf[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        qk_group(gidx, kf[gidx & 1]);
+        exp_chunk(sc, gidx - 1, m_use, pb[gidx - 1]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // the first output products under the last exponentials
+      read_v(Vb, 1, vf[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      pv_step(vf[0], pb[0]);
+      exp_chunk(sc, NPS - 1, m_use, pb[NPS - 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int sidx = 1; sidx < NPS; ++sidx) {
+        if (sidx + 1 < NPS) read_v(Vb, sidx + 1, vf[(sidx + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        pv_step(vf[sidx & 1], pb[sidx]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      JV_PRIO(0);
+    };
+
+    // Every live wave takes every tile the block walks (a tile it sees nothing of is masked like any
+    // other: at most one per block when neighbouring groups are paired): one path through the loop.
+    f32x16 sa[2], sb[2];
+    int j0 = j_first, j1 = next_tile(j0), j2 = j1 < kv_end ? next_tile(j1) : j1;
+    unsigned pga[PCS], pgb[PCS];
+    pages_of(j0, pga);
+    fetch_k(0, pga);
+    fetch_v(0, pga);
+    if (j1 < kv_end) {
+      pages_of(j1, pga);
+      fetch_k(1, pga);                                // pga: the pages of tile 1, whose V is fetched in the first turn
+    }
+    if (j2 < kv_end) pages_of(j2, pgb);
+    arrived();
+    if (j0 + BN > kv_end) fix_tail(j0, 0);
+    __syncthreads();
+    if (wave_live) tile_qk(sa, Ks[0]);
+    // one turn: tile t (scores in sc, K and V in buffers b), tile t + 1 (scores into sn, K in buffer b ^ 1)
+    auto turn = [&](f32x16 (&sc)[2], f32x16 (&sn)[2], int b) {
+      const bool has2 = j2 < kv_end;
+      fetch_v(b ^ 1, pga);                            // V(t+1) where V(t-1) was
+      if (has2) fetch_k(b, pgb);                      // K(t+2) where K(t) was: its scores were made in the last turn
+      const int j3 = has2 ? next_tile(j2) : j2;
+#pragma unroll
+      for (int i = 0; i < PCS; ++i) pga[i] = pgb[i];
+      if (j3 < kv_end) pages_of(j3, pgb);
+      if (wave_live) tile_both(sc, sn, j0, Ks[b ^ 1], Vs[b]);
+      arrived();
+      if (j1 + BN > kv_end) fix_tail(j1, b ^ 1);
+      __syncthreads();
+      j0 = j1; j1 = j2; j2 = j3;
+    };
+    int b = 0;
+    while (j1 < kv_end) {
+      turn(sa, sb, 0);
+      b = 1;
+      if (j1 >= kv_end) break;
+      turn(sb, sa, 1);
+      b = 0;
+    }
+    if (wave_live) {                                  // the last tile: nothing follows it
+      if (b == 0) tile_sm(sa, j0, Vs[0]);
+      else tile_sm(sb, j0, Vs[1]);
+    }
+  } else {
   unsigned pg[PCS];
   if (FAST) {
     pages_of(j_first, pg);
@@ -875,6 +1102,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     j0 = j_next;
     b ^= 1;
+  }
   }
 
   float l = l_lane + __shfl_xor(l_lane, 32, 64);
@@ -1184,7 +1412,7 @@ extern "C" int jv_attn_prefill(void* out, const void* q, long long q_row_stride,
   const int mode = (a.page_shift >= 3 && a.page_shift <= 6) ? 1 : (a.page_shift > 6 ? 2 : 0);
 #ifdef JV_PREFILL32
   constexpr bool pow2 = (D & (D - 1)) == 0;
-  void (*kernel)(AttnArgs) = (page_size == 16 && pow2) ? attn_prefill32_kernel<pow2 ? 16 : 1>
+  void (*kernel)(AttnArgs) = (page_size == 16 && pow2) ? attn_prefill32_kernel<pow2 ? 16 : 1, pow2>
                              : mode == 1 ? attn_prefill32_kernel<1>
                              : mode == 2 ? attn_prefill32_kernel<2> : attn_prefill32_kernel<0>;
 #else
