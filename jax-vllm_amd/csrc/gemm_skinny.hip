@@ -338,12 +338,19 @@ static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, i
 // The next tile's weights are asked for before the current tile is multiplied and reduced.
 // A longer inner size is shared out to gridDim.y groups of blocks, 8 * NL * 32 columns each,
 // which write float partial products to y + group * M * ldy (added by the reader, in order).
-template <int NL, int MT, typename OutT, bool PAIRS>
+// No load of the loop sits inside a branch (the compiler would wrap each in a branch of its own, and wait at
+// its end): rows of W beyond N read the last row (their outputs are never stored), rows of x beyond M read
+// the last row (likewise); EDGE (the inner size is not ksplit * 8 * NL * 32 exactly): columns beyond K read
+// the row's last piece again, against zeros in x.
+template <int NL, int MT, typename OutT, bool PAIRS, bool EDGE>
 __global__ void __launch_bounds__(512)
 gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
                               int M, int N, int K, long long ldx, long long ldy) {
   y += (long long)blockIdx.y * M * ldy;
-  __shared__ __attribute__((aligned(16))) float red[8 * MT * 256];
+  // the 8 waves' partial tiles, in two buffers that take turns: one barrier per tile (the waves that do
+  // not add may run ahead into the next tile, whose partials go to the other buffer; nobody can be two
+  // tiles ahead of the adding wave, which has to pass the barrier in between)
+  __shared__ __attribute__((aligned(16))) float red[2][8 * MT * 256];
   const int tid = threadIdx.x;
   const int wk = tid >> 6, lane = tid & 63, li = lane & 15, lc = lane >> 4;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -355,31 +362,35 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
-      const int k = k0 + i * 32, m = mt * 16 + li;
-      b[mt][i] = (m < M && k < K) ? *(const bf16x8*)(x + (long long)m * ldx + k) : zero;
+      const int k = k0 + i * 32, m = min(mt * 16 + li, M - 1);
+      const bf16x8 v = *(const bf16x8*)(x + (long long)m * ldx + (EDGE ? min(k, K - 8) : k));
+      b[mt][i] = (!EDGE || k < K) ? v : zero;
     }
+  // a tile beyond the last (the prefetch after the last tile) reads the first pieces of W, the same for all lanes
   auto load_tile = [&](int tile, bf16x8 (&a)[NL]) {
-    const int n = tile * 16 + li;
-    const bf16_t* wrow = W + (long long)(n < N ? n : 0) * K + k0;
+    const int n = min(tile * 16 + li, N - 1);
+    const bool real = tile < n_tiles;
+    const bf16_t* wrow = W + (real ? (long long)n * K : 0);
+    const int kk = real ? k0 : 0;
 #pragma unroll
-    for (int i = 0; i < NL; ++i) a[i] = (n < N && k0 + i * 32 < K) ? *(const bf16x8*)(wrow + i * 32) : zero;
+    for (int i = 0; i < NL; ++i) a[i] = *(const bf16x8*)(wrow + (EDGE ? min(kk + i * 32, K - 8) : kk + i * 32));
   };
-  auto finish_tile = [&](int tile, bf16x8 (&a)[NL]) {
+  auto finish_tile = [&](int tile, bf16x8 (&a)[NL], int buf) {
     f32x4 acc[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < NL; ++i) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[mt][i], acc[mt], 0, 0, 0);
-      *(f32x4*)(red + ((wk * MT + mt) * 256 + lane * 4)) = acc[mt];
+      *(f32x4*)(red[buf] + ((wk * MT + mt) * 256 + lane * 4)) = acc[mt];
     }
     __syncthreads();
     if (wk < MT) {                                 // wave mt adds row tile mt, in fixed order: wave 0, 1, ..., 7
       const int mt = wk;
-      f32x4 s = *(const f32x4*)(red + (mt * 256 + lane * 4));
+      f32x4 s = *(const f32x4*)(red[buf] + (mt * 256 + lane * 4));
 #pragma unroll
       for (int w = 1; w < 8; ++w) {
-        const f32x4 t = *(const f32x4*)(red + ((w * MT + mt) * 256 + lane * 4));
+        const f32x4 t = *(const f32x4*)(red[buf] + ((w * MT + mt) * 256 + lane * 4));
         s[0] += t[0]; s[1] += t[1]; s[2] += t[2]; s[3] += t[3];
       }
       const int nb = tile * 16 + lc * 4;           // the accumulator holds y^T[n = lc*4+e][m = mt*16 + li]
@@ -397,20 +408,27 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
         }
       }
     }
-    __syncthreads();                               // red may be written again
   };
+  // The next tile's weights are asked for before this tile is multiplied, without a condition (beyond the
+  // last tile the last one is read again): after a conditional prefetch the compiler must assume that
+  // nothing younger is in flight, and its wait for this tile's first piece then waits for the prefetch too.
   bf16x8 a0[NL], a1[NL];
-  int tile = blockIdx.x;
-  if (tile < n_tiles) load_tile(tile, a0);
-  while (tile < n_tiles) {
+  int tile = blockIdx.x;                             // the launch has no more blocks than tiles
+  load_tile(tile, a0);
+  for (;;) {
     int next = tile + gridDim.x;
-    if (next < n_tiles) load_tile(next, a1);
-    finish_tile(tile, a0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_tile(next, a1);
+    __builtin_amdgcn_sched_barrier(0);
+    finish_tile(tile, a0, 0);
+    if (next >= n_tiles) break;
     tile = next;
-    if (tile >= n_tiles) break;
     next = tile + gridDim.x;
-    if (next < n_tiles) load_tile(next, a0);
-    finish_tile(tile, a1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_tile(next, a0);
+    __builtin_amdgcn_sched_barrier(0);
+    finish_tile(tile, a1, 1);
+    if (next >= n_tiles) break;
     tile = next;
   }
 }
@@ -421,8 +439,12 @@ static int launch_persistent(void* y, const void* x, const void* W, int M, int N
   const int n_tiles = (N + 15) / 16;
   blocks = (blocks + ksplit - 1) / ksplit;           // per group
   if (blocks > n_tiles) blocks = n_tiles;
-  hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS>), dim3(blocks, ksplit), dim3(512), 0,
-                     stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
+  if (K == ksplit * 8 * NL * 32)
+    hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, false>), dim3(blocks, ksplit), dim3(512), 0,
+                       stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
+  else
+    hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, true>), dim3(blocks, ksplit), dim3(512), 0,
+                       stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
   return JV_LAUNCH_CHECK();
 }
 

@@ -1155,16 +1155,20 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
   const int g = blockIdx.y / mt_per_head, mt = blockIdx.y - g * mt_per_head;
   const int split = blockIdx.z;
   const int* gtable = p.block_tables + (long long)r * p.table_stride;
+  // A table row beyond DEC_TBL_MAX entries does not fit: the block then copies only the entries of its own
+  // split's keys, once it knows them (one more round trip, at contexts where that does not matter; the
+  // entry point makes sure that a split's entries fit).  Pages are always looked up in LDS: a lookup in
+  // global memory beside it would be a load inside a branch, at whose end the compiler waits for every
+  // load in flight, tile after tile.
   int* tbl = (int*)(smem + 4 * (32 + 16 * D));
-  const bool table_in_lds = p.table_stride <= DEC_TBL_MAX;
-  if (table_in_lds)
+  const bool whole_row = p.table_stride <= DEC_TBL_MAX;
+  if (whole_row)
     for (int i = tid; i < p.table_stride; i += 256) tbl[i] = gtable[i];
   const int tok = p.cu_seqlens ? p.cu_seqlens[r] : r;
   const int pos = p.context_lens[r];      // the query's position; keys 0..pos are stored
   const int kv_len = pos + 1;
   int kv_begin = 0;
   if (p.window > 0 && pos - p.window + 1 > 0) kv_begin = pos - p.window + 1;
-  auto page_at = [&](int idx) -> long long { return table_in_lds ? tbl[idx] : gtable[idx]; };
 
   const int hg = mt * 16 + li;
   const bool row_ok = hg < G;
@@ -1191,19 +1195,32 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  __syncthreads();   // the table row is in LDS
+  int tbl_first = 0;                      // table entry that tbl[0] holds
+  if (!whole_row && t_lo < t_hi) {
+    tbl_first = ps.index(t_lo * BND);
+    const int j_last = (t_hi * BND < kv_len ? t_hi * BND : kv_len) - 1;
+    int n = ps.index(j_last) - tbl_first + 1;
+    if (n > DEC_TBL_MAX) n = DEC_TBL_MAX;             // never, by the entry point's check
+    for (int i = tid; i < n; i += 256) tbl[i] = gtable[tbl_first + i];
+  }
+  __syncthreads();   // the table entries are in LDS
+  auto page_at = [&](int idx) -> long long { return tbl[idx - tbl_first]; };
   // One tile's operands, global -> registers.  Nothing here looks at a loaded value, so a tile's
   // loads are in flight while the tile before it is multiplied.  Keys at or past kv_len read the
   // null page: their scores are masked by position, their V entries are zeroed before use.
   //   K operand: lane (key li of sub-tile kt, chunk lc) <- 8 consecutive d of that key
   //   V^T operand: lane (d = dt*16 + li, chunk lc) <- keys kt*16 + lc*4 .. +4 of that d
-  auto load_tile = [&](int t, bf16x8 (&kf)[2][NKS], bf16x4 (&vf)[2][NDT]) {
+  // `real` false (the prefetch behind the wave's last tile): everything is read from the null page.  The
+  // prefetch is never skipped: after a conditional one the compiler must assume that nothing younger is
+  // in flight, and its waits for this tile's operands would wait for the prefetched tile as well.
+  auto load_tile = [&](int t, bool real, bf16x8 (&kf)[2][NKS], bf16x4 (&vf)[2][NDT]) {
     const int j0 = t * BND;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       const int j = j0 + kt * 16 + li;
-      const bool ok = j < kv_len;
-      const long long page = ok ? page_at(ps.index(j)) : 0;
+      const bool ok = real && j < kv_len;
+      const long long looked = page_at(ok ? ps.index(j) : tbl_first);
+      const long long page = ok ? looked : 0;
       const bf16_t* krow = p.k_pages + ((page * p.nkv + g) * P + (ok ? ps.slot(j) : 0)) * (long long)D;
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
@@ -1214,8 +1231,9 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       const int j = j0 + kt * 16 + lc * 4;
-      const bool ok = j < kv_len;
-      const long long page = ok ? page_at(ps.index(j)) : 0;
+      const bool ok = real && j < kv_len;
+      const long long looked = page_at(ok ? ps.index(j) : tbl_first);
+      const long long page = ok ? looked : 0;
       const bf16_t* vbase = p.v_pages + (page * p.nkv + g) * (long long)D * P + (ok ? ps.slot(j) : 0);
 #pragma unroll
       for (int dt = 0; dt < NDT; ++dt) vf[kt][dt] = *(const bf16x4*)(vbase + (long long)(dt * 16 + li) * P);
@@ -1286,13 +1304,17 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_decode_kernel(Attn
     bf16x8 kf_a[2][NKS], kf_b[2][NKS];
     bf16x4 vf_a[2][NDT], vf_b[2][NDT];
     int t = t_lo + wave;
-    if (t < t_hi) load_tile(t, kf_a, vf_a);
+    load_tile(t, t < t_hi, kf_a, vf_a);
     while (t < t_hi) {
-      if (t + 4 < t_hi) load_tile(t + 4, kf_b, vf_b);
+      __builtin_amdgcn_sched_barrier(0);
+      load_tile(t + 4, t + 4 < t_hi, kf_b, vf_b);
+      __builtin_amdgcn_sched_barrier(0);
       multiply(t, kf_a, vf_a);
       t += 4;
       if (t >= t_hi) break;
-      if (t + 4 < t_hi) load_tile(t + 4, kf_a, vf_a);
+      __builtin_amdgcn_sched_barrier(0);
+      load_tile(t + 4, t + 4 < t_hi, kf_a, vf_a);
+      __builtin_amdgcn_sched_barrier(0);
       multiply(t, kf_b, vf_b);
       t += 4;
     }
@@ -1392,6 +1414,8 @@ static int check_common(AttnArgs& a) {
 }
 
 extern "C" int jv_attn_head_dim() { return D; }
+extern "C" int jv_attn_decode_table_entries() { return DEC_TBL_MAX; }
+extern "C" int jv_attn_decode_tile_keys() { return BND; }
 
 extern "C" int jv_attn_prefill(void* out, const void* q, long long q_row_stride, const void* k_pages,
                                const void* v_pages, const int* block_tables, int table_stride,
@@ -1449,8 +1473,15 @@ extern "C" int jv_attn_decode(void* out, const void* q, long long q_row_stride, 
   }
   const int G = nq / nkv, mt_per_head = (G + 15) / 16;
   if ((long long)nkv * mt_per_head > 65535 || a.num_splits > 65535) return (int)hipErrorInvalidValue;
+  // a table row that does not fit in LDS whole: every split's own entries must (keys of a split span at most
+  // ceil(tiles / splits) tiles of BND keys, hence that many keys over the page size, plus the pages it cuts)
+  if (table_stride > DEC_TBL_MAX) {
+    const long long tiles = ((long long)table_stride * page_size + BND - 1) / BND;
+    const long long per_split = (tiles + a.num_splits - 1) / a.num_splits;
+    if (per_split * BND / page_size + 2 > DEC_TBL_MAX) return (int)hipErrorInvalidValue;
+  }
   const size_t shmem = 4 * (32 + 16 * D) * sizeof(float) +
-                       (table_stride <= DEC_TBL_MAX ? (size_t)table_stride * sizeof(int) : 0);
+                       (size_t)(table_stride <= DEC_TBL_MAX ? table_stride : DEC_TBL_MAX) * sizeof(int);
   if (shmem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)attn_decode_kernel,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);

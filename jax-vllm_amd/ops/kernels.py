@@ -414,9 +414,9 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     measured on MI355X at the matrix shapes of 8B-, 14B- and 32B-class models (pure reads of the
     same bytes: 33 MB 6.5 us, 50 MB 9.1, 101 MB 16.5, 201 MB 33.5).
 
-    * wide matrices (>= 1,024 row tiles), inner size <= 4,096, 3..16 rows: blocks that stay, one per
-      compute unit (two for very wide ones), x in registers: 201 MB in 38 us at 8 rows and 40.5 at
-      16, against 42 and 53 with x staged per block, 44 by the library;
+    * wide matrices (>= 1,024 row tiles), inner size <= 4,096, up to 16 rows: blocks that stay, one per
+      compute unit (two for very wide ones), x in registers: 201 MB in 36.7 us at 8 rows, 36.2 at one
+      row, against 42 and 38.5 with x staged per block, 44 by the library;
     * narrow matrices whose reader adds partial products, up to 16 rows: the inner size shared out
       to 4 groups so that ~1,000 blocks stream (33 MB: 8.6 us against 11.0 from 256 blocks); staying
       blocks at inner sizes up to 4,096 and where a group's share is long (4,096 x 12,288 at 8 rows:
@@ -429,7 +429,8 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
       staying blocks with two row tiles of x in registers, the inner size shared out to 4 groups
       (4,096 x 4,096 at 32 rows: 10.8 us against the library's 13.0; at 33..64 rows the four row
       tiles pull x through the caches too often: the library's);
-    * one or two rows against wide matrices: x resident in LDS (chosen inside the kernel library);
+    * one or two rows against very wide matrices (the output embedding): x resident in LDS (chosen
+      inside the kernel library; 1.24 GB in 202 us against 205);
     * 9..16 rows of a large matrix that fits none of these: the library (its wider tiles amortise
       x), unless the inner size is beyond 12,288, where the library needs 113 us for the 178 MB
       that x resident in LDS streams in 45;
@@ -460,7 +461,7 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
             fewer = _fit_parts(-(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32)), parts)
             if fewer > 1 and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX and k <= LIBRARY_MAX_INNER):
                 return PARTIAL_SHAPE, fewer
-    if m >= 3 and tiles >= 4 * cus:
+    if tiles >= 4 * cus and (m >= 3 or tiles < 16 * cus):
         nl = _stay_pieces(k, 1)
         if nl is not None:
             return (-2, (2 if tiles >= 16 * cus else 1) * cus, nl), 1
@@ -552,9 +553,10 @@ def _attention_library(head_dim: int):
     if head_dim not in _checked_attention_libraries:
         lib.jv_attn_decode_scratch_floats.restype = c_longlong
         got = (lib.jv_attn_head_dim(), lib.jv_attn_prefill_group_rows(), lib.jv_attn_prefill_groups_per_item(),
-               bool(lib.jv_attn_prefill_waves_split()), lib.jv_attn_decode_scratch_floats(c_int(3), c_int(5), c_int(7)))
+               bool(lib.jv_attn_prefill_waves_split()), lib.jv_attn_decode_scratch_floats(c_int(3), c_int(5), c_int(7)),
+               lib.jv_attn_decode_table_entries(), lib.jv_attn_decode_tile_keys())
         want = (head_dim, *attn_prefill_geometry(head_dim), attn_prefill_waves_split(head_dim),
-                attn_decode_scratch_floats(3, 5, 7, head_dim))
+                attn_decode_scratch_floats(3, 5, 7, head_dim), ATTN_DECODE_TABLE_ENTRIES, ATTN_DECODE_TILE_KEYS)
         if got != want:
             raise KernelArgumentError(f"attention library for head size {head_dim} reports {got}, the planner expects {want}")
         _checked_attention_libraries.add(head_dim)
@@ -608,6 +610,21 @@ def attn_prefill_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_s
     )
 
 
+ATTN_DECODE_TABLE_ENTRIES = 4096    # page-table entries a block of the decode kernel keeps in LDS
+ATTN_DECODE_TILE_KEYS = 32          # keys of one tile of the decode kernel
+
+
+def attn_decode_min_splits(table_width: int, page_size: int) -> int:
+    """The fewest splits with which the decode kernel takes block tables of this width: a row of up to
+    4,096 entries is kept in LDS whole; of a wider one a block keeps the entries of its own split's
+    keys, which must fit."""
+    if table_width <= ATTN_DECODE_TABLE_ENTRIES:
+        return 1
+    tiles = -(-table_width * page_size // ATTN_DECODE_TILE_KEYS)
+    tiles_per_split = (ATTN_DECODE_TABLE_ENTRIES - 2) * page_size // ATTN_DECODE_TILE_KEYS
+    return -(-tiles // tiles_per_split)
+
+
 def attn_decode_scratch_floats(n_work: int, nq: int, num_splits: int, head_dim: int) -> int:
     return n_work * nq * num_splits * (head_dim + 2) if num_splits > 1 else 0
 
@@ -625,6 +642,9 @@ def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_se
         _need(n_work == context_lens.numel() == out.shape[0], "without a work list every request has one token")
     else:
         _need(work.numel() >= n_work, "work list shorter than n_work")
+    _need(num_splits >= attn_decode_min_splits(block_tables.shape[1], page_size),
+          f"block tables of {block_tables.shape[1]} pages need at least "
+          f"{attn_decode_min_splits(block_tables.shape[1], page_size)} splits")
     if num_splits > 1:
         _need(scratch is not None and scratch.is_cuda and scratch.dtype == torch.float32
               and scratch.numel() >= attn_decode_scratch_floats(n_work, nq, num_splits, head_dim),

@@ -20,7 +20,8 @@ import torch
 
 from ..ops import kernels as K
 
-TARGET_BLOCKS = 512          # about two blocks per compute unit
+TARGET_BLOCKS = 256          # blocks of the decode kernel that fill the chip: one per compute unit (measured: 8 requests of
+                             # 1,060 keys over 8 kv heads take 14.2 us with 4 splits, 16.0 with 8; 16 requests 20.3 with 2)
 MIN_KEYS_PER_SPLIT = 128     # one 32-key tile for each of a block's 4 waves
 RESIDENT_BLOCKS = 2          # blocks of the prefill kernel that a compute unit holds at once
 
@@ -114,6 +115,9 @@ def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> Mfm
     decode = [r for r, ql in enumerate(ctx.q_lens_host) if ql == 1]
     max_kv_decode = max([ctx.context_lens_host[r] + 1 for r in decode], default=1)
     splits = decode_splits(len(decode), nkv * (-(-g // 16)), max_kv_decode) if decode else 1
+    if decode:      # a very wide block table is taken split by split
+        widest = max(t.shape[1] for t in ctx.block_tables)
+        splits = max(splits, K.attn_decode_min_splits(widest, ctx.page_size))
     decode_only = len(decode) == len(ctx.q_lens_host)       # requests 0, 1, ...: the kernel needs no list
     flat = [x for item in prefill for x in item] + ([] if decode_only else decode)
     dev = torch.tensor(flat, dtype=torch.int32).pin_memory().to(device, non_blocking=True) if flat else None

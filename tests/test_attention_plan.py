@@ -50,7 +50,8 @@ def test_window_pairs_neighbours():
 
 def test_decode_splits_fill_the_chip_but_keep_a_tile_per_wave():
     assert decode_splits(1, 8, 100) == 1                     # too few keys to share out
-    assert decode_splits(1, 8, 8192) == 64
+    assert decode_splits(1, 8, 8192) == 32                   # 8 blocks a split: 256 blocks fill the chip
+    assert decode_splits(8, 8, 1061) == 4
     assert decode_splits(64, 8, 8192) == 1                   # enough blocks already
 
 

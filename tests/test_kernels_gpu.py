@@ -570,6 +570,28 @@ def test_mfma_decode_attention(case, splits):
     assert torch.equal(again, out)
 
 
+def test_mfma_decode_attention_with_a_table_wider_than_a_block_keeps():
+    """More than 4,096 pages: a block copies only the entries of its own split's keys, so few splits are
+    refused and enough of them give the same result as everywhere else."""
+    from jax_vllm_amd.ops.kernels import KernelArgumentError, attn_decode_min_splits
+
+    nq, nkv, d, page_size = 2, 1, 16, 8
+    reqs = [(40000, 1), (33, 1), (36111, 1)]
+    scale = 1.0 / math.sqrt(d)
+    qs, ks, vs, dev = _mfma_inputs(nq, nkv, d, page_size, reqs, seed=11)
+    assert dev["tables"].shape[1] > 4096 and attn_decode_min_splits(dev["tables"].shape[1], page_size) == 2
+    ref = _mfma_reference(qs, ks, vs, reqs, scale, None, nq, d)
+    for splits in (2, 5, 16):
+        scratch = torch.full((K().attn_decode_scratch_floats(len(reqs), nq, splits, d),), float("nan")).cuda()
+        out = torch.full((dev["n"], nq * d), float("nan"), dtype=torch.bfloat16).cuda()
+        K().attn_decode_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                             dev["ctx"], None, len(reqs), nq, nkv, d, scale, 0, splits, scratch)
+        torch.testing.assert_close(out.double().cpu(), ref, rtol=2e-2, atol=2e-2)
+    with pytest.raises(KernelArgumentError, match="at least 2 splits"):
+        K().attn_decode_mfma(out, dev["q"], dev["stride"], dev["k_pages"], dev["v_pages"], dev["tables"], dev["cu"],
+                             dev["ctx"], None, len(reqs), nq, nkv, d, scale, 0, 1, None)
+
+
 @pytest.mark.parametrize("far_key", [0, 15, 16, 31, 32, 63, 64, 255, 256, 511, 640])
 @pytest.mark.parametrize("kernel", ["prefill", "decode1", "decode5"])
 def test_mfma_attention_finds_one_far_key(kernel, far_key):
