@@ -448,7 +448,7 @@ static int launch_persistent(void* y, const void* x, const void* W, int M, int N
   return JV_LAUNCH_CHECK();
 }
 
-// wr == -2: nks = NL in {4, 5, 8, 10, 12, 16, 17}, wk = blocks in all; the inner size must be at most
+// wr == -2: nks = NL in {4, 5, 8, 10, 12, 16, 17, 20}, wk = blocks in all; the inner size must be at most
 // ksplit * 8 * NL * 32 and more than (ksplit - 1) * 8 * NL * 32.  Up to 16 rows with every NL, up
 // to 32 rows (two row tiles of x in registers) with NL <= 8.
 template <typename OutT, bool PAIRS>
@@ -473,6 +473,7 @@ static int dispatch_persistent(int nl, void* y, const void* x, const void* W, in
     case 12: return launch_persistent<12, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
     case 16: return launch_persistent<16, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
     case 17: return launch_persistent<17, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 20: return launch_persistent<20, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
   }
   return (int)hipErrorInvalidValue;
 }

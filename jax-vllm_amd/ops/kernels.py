@@ -383,7 +383,7 @@ def compute_units(device) -> int:
     return n
 
 
-STAY_PIECES = (4, 5, 8, 10, 12, 16, 17)   # weight pieces per wave the staying blocks are built for
+STAY_PIECES = (4, 5, 8, 10, 12, 16, 17, 20)   # weight pieces per wave the staying blocks are built for
 
 
 def _fit_parts(units: int, parts: int) -> int:
@@ -408,7 +408,8 @@ TILE64_MIN_SHARE = 3072             # columns a block of gemm_tile64 needs to pa
 LIBRARY_MAX_INNER = 12288           # beyond this inner size the library's choice for few rows collapses
 
 
-def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok: bool = False, device=None):
+def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok: bool = False, device=None,
+                   partial_max_width: int | None = PARTIAL_SUM_MAX_WIDTH):
     """How ``linear`` runs a bfloat16 product at few rows: (block_shape, ksplit) for ``gemm_skinny``
     (``TILE64`` as block shape: for ``gemm_tile64``), or None for the library.  All thresholds are
     measured on MI355X at the matrix shapes of 8B-, 14B- and 32B-class models (pure reads of the
@@ -419,9 +420,9 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
       row, against 42 and 38.5 with x staged per block, 44 by the library;
     * narrow matrices whose reader adds partial products, up to 16 rows: the inner size shared out
       to 4 groups so that ~1,000 blocks stream (33 MB: 8.6 us against 11.0 from 256 blocks); staying
-      blocks at inner sizes up to 4,096 and where a group's share is long (4,096 x 12,288 at 8 rows:
-      21.1 us against 24.9 with x resident in LDS, at 16 rows 22.1 against 30.4; 5,120 x 17,408:
-      36.4 against 40.8), x resident in LDS otherwise (5,120 x 8,192: 21.0 against 22.8);
+      blocks wherever a piece count fits the inner size (4,096 x 12,288 at 8 rows: 20.7 us against 24.9
+      with x resident in LDS; 5,120 x 17,408: 35.9 against 40.8; 5,120 x 8,192: 17.9 against 20.0), x
+      resident in LDS otherwise (5,120 x 25,600, which would need more than 4 groups);
     * the same at 17..64 rows when every block gets at least 3,072 columns: blocks of 64 rows of w,
       one per compute unit (the feed-forward's second product: 4,096 x 12,288 at 64 rows 30 us
       against the library's 37; 5,120 x 17,408 65 against 131; 5,120 x 25,600 91 against 157);
@@ -439,7 +440,7 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     if k % 8:
         return None
     cus = compute_units(device) if device is not None else 256
-    narrow = partial_ok and not silu_pairs and n % 4 == 0 and n <= PARTIAL_SUM_MAX_WIDTH
+    narrow = partial_ok and not silu_pairs and n % 4 == 0 and (partial_max_width is None or n <= partial_max_width)
     if m > SKINNY_AUTO_ROWS:
         if narrow and m <= SKINNY_MAX_ROWS:
             parts = _fit_parts(-(-k // 256), min(4, cus // -(-n // 64)))
@@ -450,14 +451,17 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
                 return (-2, cus, nl), 4
         return None
     tiles = -(-n // 16)
-    if narrow and tiles * 2 <= PARTIAL_BLOCKS:
+    if narrow and tiles <= PARTIAL_BLOCKS:
+        for parts in (4, 2):                       # staying blocks: the more groups, the fewer registers hold x
+            nl = _stay_pieces(k, parts)
+            if nl is not None:
+                # up to 8 pieces two blocks fit a compute unit, which pays up to an inner size of 4,096; beyond,
+                # one block each walks its tiles (7,168 x 5,120 at 8 rows: 16.4 us against 16.9, and against
+                # 18.9 with x resident in LDS; 5,120 x 8,192: 17.9 against 19.9 and 20.0)
+                return (-2, (2 if nl <= 8 and k <= 4096 else 1) * cus, nl), parts
         parts = min(4, -(-PARTIAL_BLOCKS // tiles))
         parts = 4 if parts == 3 else parts
         if parts > 1:
-            nl = _stay_pieces(k, parts)
-            if nl is not None and (k <= 4096 or nl >= 12 or m > 8):
-                # up to 8 pieces two blocks fit a compute unit; beyond, one block each walks its tiles
-                return (-2, (2 if nl <= 8 else 1) * cus, nl), parts
             fewer = _fit_parts(-(-k // (PARTIAL_SHAPE[1] * PARTIAL_SHAPE[2] * 32)), parts)
             if fewer > 1 and not (m > 8 and n * k >= SKINNY_LARGE_MATRIX and k <= LIBRARY_MAX_INNER):
                 return PARTIAL_SHAPE, fewer
@@ -470,7 +474,8 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     return (0, 0, 0), 1
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = False, silu_pairs: bool = False):
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = False, silu_pairs: bool = False,
+           partial_max_width: int | None = PARTIAL_SUM_MAX_WIDTH):
     """x @ w.T for w stored [out, in].
 
     float32: the library's own float-FMA kernel (no reduced-precision matrix mode).
@@ -478,7 +483,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
     library (``streaming_plan``).
     bfloat16 otherwise: a plain library matrix product (hipBLASLt through torch), float accumulation.
     With ``partial_ok`` the caller takes a float32 stack [parts, M, N] of partial products as well
-    (to be added in order, as ``add_rmsnorm`` does); it is returned for narrow matrices at up to 64 rows.
+    (to be added in order, as ``add_rmsnorm`` does); it is returned for narrow matrices at up to 64 rows
+    (``partial_max_width``: the widest row whose parts the caller's reader adds; None: any).
     With ``silu_pairs`` the rows of w alternate gate and up rows and the result is
     silu(x.w[2j]) * (x.w[2j+1]) of width N/2 (an epilogue of the streaming kernels, a kernel of
     its own after the library's product).
@@ -488,7 +494,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
     else:
         _need(x.dtype == w.dtype, "x and w must have one type")
         plan = streaming_plan(x.shape[0], w.shape[0], w.shape[1], silu_pairs,
-                              partial_ok and out_dtype in (None, torch.bfloat16), x.device)
+                              partial_ok and out_dtype in (None, torch.bfloat16), x.device, partial_max_width)
         if plan is not None:
             shape, parts = plan
             if shape == TILE64:

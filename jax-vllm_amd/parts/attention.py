@@ -76,8 +76,8 @@ class GroupedQueryAttention:
             self.position.fused_arguments(ctx) if self.position is not None else (None, 0, False)
         )
         # at few rows the projection may come as float partial products, which the next kernel adds
-        qkv = K.linear(x, self.w_qkv, partial_ok=K.rope_takes_parts(x.dtype, self.d, interleaved, rotary_dim,
-                                                                    cos_sin is not None))
+        qkv = K.linear(x, self.w_qkv, partial_max_width=None,       # the rotation kernel adds parts of any width
+                       partial_ok=K.rope_takes_parts(x.dtype, self.d, interleaved, rotary_dim, cos_sin is not None))
         parts = None
         if qkv.dim() == 3:
             parts, qkv = qkv, torch.empty(qkv.shape[1:], dtype=x.dtype, device=x.device)

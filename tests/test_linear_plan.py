@@ -62,5 +62,11 @@ def test_plans_at_the_sizes_they_were_measured_at():
     assert plan(64, 4096, 4096, partial_ok=True) is None                        # short inner size: the library's
     assert plan(32, 4096, 4096, partial_ok=True) == ((-2, 256, 4), 4)           # two row tiles of x in registers
     assert plan(12, 5120, 17408, partial_ok=True) == ((-2, 256, 17), 4)         # where the library collapses
-    assert plan(8, 1024, 3072, partial_ok=True)[1] == 3                         # 6 phases do not share out to 4 groups
+    assert plan(8, 1024, 3072, partial_ok=True) == ((-2, 512, 8), 2)            # no piece count covers 3,072 with 4 groups
+    assert plan(8, 5120, 25600, partial_ok=True) == (K.PARTIAL_SHAPE, 4)        # none with 2 or 4: x resident in LDS
+    assert plan(8, 1024, 1000 * 8, partial_ok=True)[1] in (2, 3, 4)
+    assert plan(8, 34816, 5120, silu_pairs=True) == ((-2, 256, 20), 1)          # gate and up, 14B
+    assert plan(1, 24576, 4096, silu_pairs=True) == ((-2, 256, 16), 1)          # one row: the same blocks
+    assert plan(8, 10240, 5120, partial_ok=True) == ((0, 0, 0), 1)              # wider than the norm adds parts of ...
+    assert plan(8, 10240, 5120, partial_ok=True, partial_max_width=None) == ((-2, 256, 5), 4)   # ... but the rotation kernel does
     assert plan(8, 4096, 4100) is None                                          # inner size no multiple of 8
