@@ -454,9 +454,23 @@ static int launch_persistent(void* y, const void* x, const void* W, int M, int N
 template <typename OutT, bool PAIRS>
 static int dispatch_persistent(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
                                long long ldy, int blocks, int ksplit, hipStream_t s) {
-  if (M > 32 || (M > 16 && nl > 8) || blocks < 1 || ksplit > 65535 || K > (long long)ksplit * 8 * nl * 32 ||
-      K <= (long long)(ksplit - 1) * 8 * nl * 32)
+  if (M > 64 || (M > 16 && nl > 8) || (M > 32 && nl > 5) || blocks < 1 || ksplit > 65535 ||
+      K > (long long)ksplit * 8 * nl * 32 || K <= (long long)(ksplit - 1) * 8 * nl * 32)
     return (int)hipErrorInvalidValue;
+  if (M > 48) {
+    switch (nl) {
+      case 4: return launch_persistent<4, 4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+      case 5: return launch_persistent<5, 4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    }
+    return (int)hipErrorInvalidValue;
+  }
+  if (M > 32) {
+    switch (nl) {
+      case 4: return launch_persistent<4, 3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+      case 5: return launch_persistent<5, 3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    }
+    return (int)hipErrorInvalidValue;
+  }
   if (M > 16) {
     switch (nl) {
       case 4: return launch_persistent<4, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);

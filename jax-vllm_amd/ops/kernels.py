@@ -311,7 +311,7 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     _need(m <= SKINNY_MAX_ROWS, f"gemm_skinny takes at most {SKINNY_MAX_ROWS} rows")
     _need(k % 8 == 0, "the inner size must be a multiple of 8")
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
-    _need(block_shape[0] != -2 or ((m <= 16 or (m <= 32 and block_shape[2] <= 8)) and block_shape[2] in STAY_PIECES
+    _need(block_shape[0] != -2 or ((m <= 16 or (m <= 32 and block_shape[2] <= 8) or block_shape[2] <= 5) and block_shape[2] in STAY_PIECES
                                    and 256 * block_shape[2] * (ksplit - 1) < k <= 256 * block_shape[2] * ksplit),
           "the organisation with blocks that stay takes at most 16 rows (32 with at most 8 pieces) and an inner "
           "size of ksplit * 256 * pieces at most")
@@ -426,10 +426,11 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     * the same at 17..64 rows when every block gets at least 3,072 columns: blocks of 64 rows of w,
       one per compute unit (the feed-forward's second product: 4,096 x 12,288 at 64 rows 30 us
       against the library's 37; 5,120 x 17,408 65 against 131; 5,120 x 25,600 91 against 157);
-    * 17..32 rows against narrow matrices with a short inner size (the attention's output product):
-      staying blocks with two row tiles of x in registers, the inner size shared out to 4 groups
-      (4,096 x 4,096 at 32 rows: 10.8 us against the library's 13.0; at 33..64 rows the four row
-      tiles pull x through the caches too often: the library's);
+    * 17..64 rows against narrow matrices with a short inner size (the attention's products): staying
+      blocks, one per compute unit, with two to four row tiles of x in registers (up to 8 pieces a
+      wave for two, 5 for more), the inner size shared out to 4 groups (4,096 x 4,096: 10.3 us at
+      32 rows, 13.2 at 64, against the library's 13.0 and 15.0; 5,120 x 5,120 at 48 rows: 16.5
+      against 26.6);
     * one or two rows against very wide matrices (the output embedding): x resident in LDS (chosen
       inside the kernel library; 1.24 GB in 202 us against 205);
     * 9..16 rows of a large matrix that fits none of these: the library (its wider tiles amortise
@@ -447,7 +448,7 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
             if parts >= 2 and k >= parts * TILE64_MIN_SHARE:
                 return TILE64, parts
             nl = _stay_pieces(k, 4)
-            if m <= 32 and nl is not None and nl <= 8 and -(-n // 16) * 2 <= PARTIAL_BLOCKS:
+            if nl is not None and -(-n // 16) * 2 <= PARTIAL_BLOCKS and (nl <= 5 or (m <= 32 and nl <= 8)):
                 return (-2, cus, nl), 4
         return None
     tiles = -(-n // 16)

@@ -724,7 +724,7 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     (1, 8200, 4096, (0, 0, 0)), (2, 100, 4096, (-1, 8, 16)), (8, 333, 1000, (-1, 16, 4)), (16, 64, 12288, (-1, 4, 8)),
     (11, 50, 72, (-1, 3, 4)), (8, 24576, 512, (-2, 64, 4)), (16, 333, 4096, (-2, 7, 16)), (5, 777, 2000, (-2, 1000, 8)),
     (3, 100, 72, (-2, 3, 4)), (1, 8200, 4096, (-2, 256, 16)), (17, 333, 1000, (-2, 40, 4)), (32, 4096, 2048, (-2, 256, 8)),
-    (25, 50, 1200, (-2, 9, 5))])
+    (25, 50, 1200, (-2, 9, 5)), (40, 333, 1000, (-2, 40, 4)), (64, 200, 1280, (-2, 30, 5)), (49, 77, 1016, (-2, 3, 4)), (8, 200, 4904, (-2, 16, 20))])
 def test_gemm_skinny(m, n, k, shape, out_dtype):
     x = randn(m, k, dtype=torch.bfloat16, seed=30, scale=0.5)
     w = randn(n, k, dtype=torch.bfloat16, seed=31, scale=0.5)
@@ -747,7 +747,8 @@ def test_gemm_skinny(m, n, k, shape, out_dtype):
                                                 (16, 333, 1000, (-1, 8, 2), 2), (5, 64, 2560, (-1, 4, 4), 3),
                                                 (3, 48, 1000, (-1, 2, 2), 4), (8, 4096, 4096, (-2, 512, 4), 4),
                                                 (16, 130, 3000, (-2, 10, 4), 3), (2, 64, 12288, (-2, 30, 16), 3),
-                                                (32, 4096, 4096, (-2, 256, 4), 4), (20, 136, 5120, (-2, 33, 5), 4)])
+                                                (32, 4096, 4096, (-2, 256, 4), 4), (20, 136, 5120, (-2, 33, 5), 4),
+                                                (64, 520, 4096, (-2, 256, 4), 4), (41, 136, 4800, (-2, 7, 5), 4)])
 def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
     """Partial products [ksplit, M, N] in float: part s covers its own columns only, and the
     ordered sum is the product."""
@@ -831,7 +832,8 @@ def test_linear_takes_blocks_of_64_rows_for_a_long_inner_size():
     plan = kern.streaming_plan(m, n, k, partial_ok=True, device=x.device)
     assert plan == (kern.TILE64, 4)
     assert kern.streaming_plan(m, n, k, partial_ok=False, device=x.device) is None
-    assert kern.streaming_plan(m, n, 4096, partial_ok=True, device=x.device) is None      # too few columns a block
+    assert kern.streaming_plan(m, n, 4096, partial_ok=True, device=x.device) == ((-2, 256, 4), 4)   # too few columns a block of 64 rows: staying blocks
+    assert kern.streaming_plan(m, n, 8192, partial_ok=True, device=x.device) is None      # ... unless x would not fit their registers
     few = kern.streaming_plan(12, 5120, 17408, partial_ok=True, device=x.device)     # not the library's either
     assert few is not None and few[1] == 4 and few[0][0] in (-1, -2)
     parts = kern.linear(x, w, partial_ok=True)

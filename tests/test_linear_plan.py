@@ -26,7 +26,7 @@ def acceptable(m, n, k, silu, plan):
         return "more than 64 rows"
     kind, a, b = shape
     if kind == -2:
-        if (m > 16 and (m > 32 or b > 8)) or b not in K.STAY_PIECES or a < 1 or \
+        if (m > 16 and b > 8) or (m > 32 and b > 5) or b not in K.STAY_PIECES or a < 1 or \
                 not (256 * b * (parts - 1) < k <= 256 * b * parts):
             return "staying blocks that do not cover the inner size"
     elif kind == -1:
@@ -59,7 +59,8 @@ def test_plans_at_the_sizes_they_were_measured_at():
     assert plan(8, 24576, 4096, silu_pairs=True) == ((-2, 256, 16), 1)          # gate and up, 8B
     assert plan(64, 4096, 12288, partial_ok=True) == (K.TILE64, 4)              # down_proj at 64 rows
     assert plan(64, 5120, 17408, partial_ok=True) == (K.TILE64, 3)              # 80 tiles of 64 rows: 3 groups fill 256 units
-    assert plan(64, 4096, 4096, partial_ok=True) is None                        # short inner size: the library's
+    assert plan(64, 4096, 4096, partial_ok=True) == ((-2, 256, 4), 4)           # four row tiles of x in registers
+    assert plan(64, 5120, 8192, partial_ok=True) is None                        # 8 pieces a wave: too many registers for that
     assert plan(32, 4096, 4096, partial_ok=True) == ((-2, 256, 4), 4)           # two row tiles of x in registers
     assert plan(12, 5120, 17408, partial_ok=True) == ((-2, 256, 17), 4)         # where the library collapses
     assert plan(8, 1024, 3072, partial_ok=True) == ((-2, 512, 8), 2)            # no piece count covers 3,072 with 4 groups
