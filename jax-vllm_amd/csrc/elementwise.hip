@@ -188,6 +188,39 @@ add_rmsnorm_parts_kernel(float* __restrict__ h, const float* __restrict__ parts,
   }
 }
 
+// The residual step of a row shared out to hidden / 512 blocks, with the norm's scale left to the reader:
+//   h[r] += parts[0][r] + parts[1][r] + ... (in that order), xg[r] = T(h[r] * w) (NOT normalised),
+//   ssq[r][b] = sum of squares of block b's 512 columns of the new h[r] (rows of 16 floats, hidden / 512 <= 16 of
+//   them written).
+// A matrix product that takes xg multiplies its output rows by rsqrt(sum_b ssq[r][b] / hidden + eps)
+// (the scale of a row commutes with the product).  One compute unit no longer has to pull a whole
+// row's five arrays: 2.3 us after a product against 3.9 for the norm kernel at 8 rows of 4,096.
+#define ARN_SHARE 512
+template <typename T, int NP>
+__global__ void __launch_bounds__(128)
+add_parts_unscaled_kernel(float* __restrict__ h, const float* __restrict__ parts, long long part_stride,
+                          const float* __restrict__ w, T* __restrict__ xg, float* __restrict__ ssq, int hidden) {
+  __shared__ float red[2];
+  const long long r = blockIdx.y;
+  const int c = blockIdx.x * (ARN_SHARE / 4) + threadIdx.x;      // 16-byte piece of the row
+  float* hr = h + r * hidden;
+  const float* pr = parts + r * hidden;
+  const float4 ww = *(const float4*)(w + 4 * c);
+  float4 v = *(const float4*)(hr + 4 * c), e[NP];
+#pragma unroll
+  for (int q = 0; q < NP; ++q) e[q] = *(const float4*)(pr + q * part_stride + 4 * c);
+  float4 d = e[0];
+#pragma unroll
+  for (int q = 1; q < NP; ++q) { d.x += e[q].x; d.y += e[q].y; d.z += e[q].z; d.w += e[q].w; }
+  v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+  *(float4*)(hr + 4 * c) = v;
+  store4<T>(xg + r * hidden + 4 * c, float4{v.x * ww.x, v.y * ww.y, v.z * ww.z, v.w * ww.w});
+  const float s = wave_sum(v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w);
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) ssq[r * 16 + blockIdx.x] = red[0] + red[1];       // rows of 16 shares, gridDim.x of them written
+}
+
 // threads of a block and 16-byte pieces per thread for a row of nvec pieces (nvec <= 8 * 256)
 static void arn_shape(int nvec, int* threads, int* v) {
   *threads = nvec >= 1024 ? 256 : (nvec >= 256 ? 128 : 64);
@@ -340,6 +373,25 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
       case 2: launch_arn_parts<T, 2>(v, n_out, vt, st, h, parts, part_stride, w, (T*)out, rows, hidden, eps); break; \
       case 3: launch_arn_parts<T, 3>(v, n_out, vt, st, h, parts, part_stride, w, (T*)out, rows, hidden, eps); break; \
       default: launch_arn_parts<T, 4>(v, n_out, vt, st, h, parts, part_stride, w, (T*)out, rows, hidden, eps); break; \
+    }                                                                                               \
+    return JV_LAUNCH_CHECK();                                                                       \
+  }                                                                                                 \
+  /* the same residual step with the norm's scale left to the reader: see add_parts_unscaled_kernel; */ \
+  /* ssq must hold n_rows * 16 floats */                                                            \
+  extern "C" int jv_add_parts_unscaled_##SUF(float* h, const float* parts, int n_parts,             \
+                                             long long part_stride, const float* w, void* xg,       \
+                                             float* ssq, int n_rows, int hidden, void* stream) {    \
+    if (n_rows <= 0) return 0;                                                                      \
+    if (n_parts < 1 || n_parts > ARN_MAX_PARTS || hidden % ARN_SHARE != 0 || n_rows > 65535 ||      \
+        hidden / ARN_SHARE > 16)                                                                    \
+      return (int)hipErrorInvalidValue;                                                             \
+    const dim3 grid(hidden / ARN_SHARE, n_rows);                                                    \
+    hipStream_t st = (hipStream_t)stream;                                                           \
+    switch (n_parts) {                                                                              \
+      case 1: hipLaunchKernelGGL((add_parts_unscaled_kernel<T, 1>), grid, dim3(128), 0, st, h, parts, part_stride, w, (T*)xg, ssq, hidden); break; \
+      case 2: hipLaunchKernelGGL((add_parts_unscaled_kernel<T, 2>), grid, dim3(128), 0, st, h, parts, part_stride, w, (T*)xg, ssq, hidden); break; \
+      case 3: hipLaunchKernelGGL((add_parts_unscaled_kernel<T, 3>), grid, dim3(128), 0, st, h, parts, part_stride, w, (T*)xg, ssq, hidden); break; \
+      default: hipLaunchKernelGGL((add_parts_unscaled_kernel<T, 4>), grid, dim3(128), 0, st, h, parts, part_stride, w, (T*)xg, ssq, hidden); break; \
     }                                                                                               \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \

@@ -338,6 +338,15 @@ static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, i
 // The next tile's weights are asked for before the current tile is multiplied and reduced.
 // A longer inner size is shared out to gridDim.y groups of blocks, 8 * NL * 32 columns each,
 // which write float partial products to y + group * M * ldy (added by the reader, in order).
+// Rows of x that come un-normalised from add_parts_unscaled_kernel: output row m is multiplied by
+// rsqrt(sum_j ssq[m][j] / width + eps), j < shares, ssq rows of 16 floats (the norm's scale commutes with the
+// product; with the inner size shared out every partial product is scaled).  ssq == nullptr: no scale.
+struct RowScale {
+  const float* ssq;
+  int shares;       // at most 16
+  float inv_width, eps;
+};
+
 // No load of the loop sits inside a branch (the compiler would wrap each in a branch of its own, and wait at
 // its end): rows of W beyond N read the last row (their outputs are never stored), rows of x beyond M read
 // the last row (likewise); EDGE (the inner size is not ksplit * 8 * NL * 32 exactly): columns beyond K read
@@ -345,7 +354,7 @@ static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, i
 template <int NL, int MT, typename OutT, bool PAIRS, bool EDGE>
 __global__ void __launch_bounds__(512)
 gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
-                              int M, int N, int K, long long ldx, long long ldy) {
+                              int M, int N, int K, long long ldx, long long ldy, RowScale rs) {
   y += (long long)blockIdx.y * M * ldy;
   // the 8 waves' partial tiles, in two buffers that take turns: one barrier per tile (the waves that do
   // not add may run ahead into the next tile, whose partials go to the other buffer; nobody can be two
@@ -367,6 +376,16 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
       b[mt][i] = (!EDGE || k < K) ? v : zero;
     }
   // a tile beyond the last (the prefetch after the last tile) reads the first pieces of W, the same for all lanes
+  // the scale of this lane's output row (wave mt adds row tile mt): asked for now, used after the first tile;
+  // without a scale the loads read x (no load inside a branch) and get no weight
+  // (one 16-byte load a lane: the 4 lanes of a row hold its 16 shares; every block reads these few lines,
+  // so every instruction more would queue up at one place in the L2)
+  f32x4 row_sq;
+  {
+    const int m = min((wk < MT ? wk : 0) * 16 + li, M - 1);
+    const float* sp = rs.ssq ? rs.ssq + (long long)m * 16 + lc * 4 : (const float*)x;
+    row_sq = *(const f32x4*)sp;
+  }
   auto load_tile = [&](int tile, bf16x8 (&a)[NL]) {
     const int n = min(tile * 16 + li, N - 1);
     const bool real = tile < n_tiles;
@@ -395,6 +414,15 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
       }
       const int nb = tile * 16 + lc * 4;           // the accumulator holds y^T[n = lc*4+e][m = mt*16 + li]
       const int m = mt * 16 + li;
+      if (rs.ssq) {                                // a fixed order of adding: the same scale in every tile and block
+        float sq = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sq += lc * 4 + j < rs.shares ? row_sq[j] : 0.f;
+        sq += __shfl_xor(sq, 16, 64);
+        sq += __shfl_xor(sq, 32, 64);
+        const float inv = rsqrtf(sq * rs.inv_width + rs.eps);
+        s[0] *= inv; s[1] *= inv; s[2] *= inv; s[3] *= inv;
+      }
       if (m < M) {
         if (PAIRS) {
 #pragma unroll
@@ -435,16 +463,16 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
 
 template <int NL, int MT, typename OutT, bool PAIRS>
 static int launch_persistent(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                             long long ldy, int blocks, int ksplit, hipStream_t stream) {
+                             long long ldy, int blocks, int ksplit, RowScale rs, hipStream_t stream) {
   const int n_tiles = (N + 15) / 16;
   blocks = (blocks + ksplit - 1) / ksplit;           // per group
   if (blocks > n_tiles) blocks = n_tiles;
   if (K == ksplit * 8 * NL * 32)
     hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, false>), dim3(blocks, ksplit), dim3(512), 0,
-                       stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
+                       stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, rs);
   else
     hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, true>), dim3(blocks, ksplit), dim3(512), 0,
-                       stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy);
+                       stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, rs);
   return JV_LAUNCH_CHECK();
 }
 
@@ -453,41 +481,41 @@ static int launch_persistent(void* y, const void* x, const void* W, int M, int N
 // to 32 rows (two row tiles of x in registers) with NL <= 8.
 template <typename OutT, bool PAIRS>
 static int dispatch_persistent(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                               long long ldy, int blocks, int ksplit, hipStream_t s) {
+                               long long ldy, int blocks, int ksplit, RowScale rs, hipStream_t s) {
   if (M > 64 || (M > 16 && nl > 8) || (M > 32 && nl > 5) || blocks < 1 || ksplit > 65535 ||
       K > (long long)ksplit * 8 * nl * 32 || K <= (long long)(ksplit - 1) * 8 * nl * 32)
     return (int)hipErrorInvalidValue;
   if (M > 48) {
     switch (nl) {
-      case 4: return launch_persistent<4, 4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-      case 5: return launch_persistent<5, 4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+      case 4: return launch_persistent<4, 4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+      case 5: return launch_persistent<5, 4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
     }
     return (int)hipErrorInvalidValue;
   }
   if (M > 32) {
     switch (nl) {
-      case 4: return launch_persistent<4, 3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-      case 5: return launch_persistent<5, 3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+      case 4: return launch_persistent<4, 3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+      case 5: return launch_persistent<5, 3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
     }
     return (int)hipErrorInvalidValue;
   }
   if (M > 16) {
     switch (nl) {
-      case 4: return launch_persistent<4, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-      case 5: return launch_persistent<5, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-      case 8: return launch_persistent<8, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+      case 4: return launch_persistent<4, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+      case 5: return launch_persistent<5, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+      case 8: return launch_persistent<8, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
     }
     return (int)hipErrorInvalidValue;
   }
   switch (nl) {
-    case 4: return launch_persistent<4, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 5: return launch_persistent<5, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 8: return launch_persistent<8, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 10: return launch_persistent<10, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 12: return launch_persistent<12, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 16: return launch_persistent<16, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 17: return launch_persistent<17, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
-    case 20: return launch_persistent<20, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, s);
+    case 4: return launch_persistent<4, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+    case 5: return launch_persistent<5, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+    case 8: return launch_persistent<8, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+    case 10: return launch_persistent<10, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+    case 12: return launch_persistent<12, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+    case 16: return launch_persistent<16, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+    case 17: return launch_persistent<17, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+    case 20: return launch_persistent<20, 1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
   }
   return (int)hipErrorInvalidValue;
 }
@@ -518,18 +546,19 @@ static void skinny_config(int M, int N, int K, int* wr, int* wk, int* nks) {
 // weight pieces per wave and phase.
 // ksplit > 1 (resident-x organisation or blocks that stay, float output only): K is shared out to ksplit blocks per
 // row tile and y is [ksplit][M][ldy], partial products that the reader adds in that order.
-extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
-                                   long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
-                                   int wk, int nks, int ksplit, void* stream) {
+static int gemm_skinny_entry(void* y, const void* x, const void* W, int M, int N, int K, long long ldx, long long ldy,
+                             int out_f32, int silu_pairs, int wr, int wk, int nks, int ksplit, RowScale rs,
+                             void* stream) {
   if (M <= 0 || N <= 0) return 0;
+  if (rs.ssq && (wr != -2 || rs.shares < 1 || rs.shares > 16)) return (int)hipErrorInvalidValue;   // only the staying blocks scale rows
   if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
   if (silu_pairs && (out_f32 || N % 2 != 0 || wr == -1)) return (int)hipErrorInvalidValue;
   if (ksplit < 1 || (ksplit > 1 && ((wr != -1 && wr != -2) || !out_f32))) return (int)hipErrorInvalidValue;
   if (wr == -2) {   // blocks that stay: wk = number of blocks, nks = weight pieces per wave
     hipStream_t s = (hipStream_t)stream;
-    if (silu_pairs) return dispatch_persistent<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s);
-    return out_f32 ? dispatch_persistent<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s)
-                   : dispatch_persistent<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s);
+    if (silu_pairs) return dispatch_persistent<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, rs, s);
+    return out_f32 ? dispatch_persistent<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, rs, s)
+                   : dispatch_persistent<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, rs, s);
   }
   if (wr == -1) {
     if (M > 16 || wk < 1 || wk > 16) return (int)hipErrorInvalidValue;
@@ -555,4 +584,22 @@ extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M,
   if (silu_pairs) return dispatch_nks<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
   if (out_f32) return dispatch_nks<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
   return dispatch_nks<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
+}
+
+extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
+                                   long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
+                                   int wk, int nks, int ksplit, void* stream) {
+  return gemm_skinny_entry(y, x, W, M, N, K, ldx, ldy, out_f32, silu_pairs, wr, wk, nks, ksplit,
+                           RowScale{nullptr, 0, 0.f, 0.f}, stream);
+}
+
+// The same for rows of x that add_parts_unscaled left un-normalised (blocks that stay only, wr == -2):
+// output row m is multiplied by rsqrt(sum_{j < shares} ssq[m * 16 + j] / width + eps).
+extern "C" int jv_gemm_skinny_scaled_bf16(void* y, const void* x, const void* W, int M, int N, int K,
+                                          long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
+                                          int wk, int nks, int ksplit, const float* ssq, int shares, int width,
+                                          float eps, void* stream) {
+  if (!ssq || width <= 0) return (int)hipErrorInvalidValue;
+  return gemm_skinny_entry(y, x, W, M, N, K, ldx, ldy, out_f32, silu_pairs, wr, wk, nks, ksplit,
+                           RowScale{ssq, shares, 1.f / (float)width, eps}, stream);
 }

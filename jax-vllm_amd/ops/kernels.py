@@ -132,6 +132,49 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out=None) -> torc
     return out
 
 
+UNSCALED_SHARE = 512          # columns of a row per block of the un-normalised residual step
+UNSCALED_MAX_SHARES = 16      # shares of a row's sum of squares that the products' epilogue adds
+
+
+class UnscaledRows:
+    """Rows ``x = h * weight`` in bfloat16 whose RMSNorm scale is still to be applied: row m of what a
+    product with them gives has to be multiplied by ``rsqrt(sum(ssq[m]) / width + eps)`` (the scale of
+    a row commutes with the product).  ``linear`` does that in the epilogue of its streaming kernels."""
+
+    def __init__(self, x: torch.Tensor, ssq: torch.Tensor, width: int, eps: float):
+        self.x, self.ssq, self.width, self.eps = x, ssq, int(width), float(eps)   # ssq [rows, 16], width / 512 of them used
+        self.shares = self.width // UNSCALED_SHARE
+
+    shape = property(lambda self: self.x.shape)
+    dtype = property(lambda self: self.x.dtype)
+    device = property(lambda self: self.x.device)
+
+
+def unscaled_rows_possible(dtype, n_rows: int, hidden: int) -> bool:
+    return (dtype == torch.bfloat16 and 0 < n_rows <= SKINNY_AUTO_ROWS and hidden % UNSCALED_SHARE == 0
+            and hidden // UNSCALED_SHARE <= UNSCALED_MAX_SHARES)
+
+
+def add_parts_unscaled(h: torch.Tensor, parts: torch.Tensor, weight: torch.Tensor, eps: float) -> "UnscaledRows":
+    """h += parts[0] + parts[1] + ... (in that order, in place, float); returns the rows h * weight in
+    bfloat16, NOT normalised, with the shares of each row's sum of squares: the residual step of a
+    decode step shared out to hidden / 512 blocks a row instead of one (the norm's reduction would
+    need the whole row in one block)."""
+    _dev(h, parts, weight)
+    _f32(h, "h")
+    n, hidden = h.shape
+    _f32(weight, "weight", hidden)
+    _need(parts.dtype == torch.float32 and parts.dim() == 3 and parts.shape[1:] == h.shape and 1 <= parts.shape[0] <= 4,
+          "partial products must be float32 [parts <= 4, *h.shape]")
+    _need(unscaled_rows_possible(torch.bfloat16, n, hidden), "at most 16 rows of a width that is a multiple of 512, at most 8192")
+    xg = torch.empty((n, hidden), dtype=torch.bfloat16, device=h.device)
+    ssq = torch.empty((n, UNSCALED_MAX_SHARES), dtype=torch.float32, device=h.device)    # hidden / 512 of a row's 16 are written
+    _check(library.core().jv_add_parts_unscaled_bf16(_ptr(h), _ptr(parts), c_int(parts.shape[0]), c_longlong(parts.stride(0)),
+                                                     _ptr(weight), _ptr(xg), _ptr(ssq), c_int(n), c_int(hidden), _stream()),
+           "add_parts_unscaled")
+    return UnscaledRows(xg, ssq, hidden, eps)
+
+
 def cast_rows(x: torch.Tensor, dtype: torch.dtype, rows=None) -> torch.Tensor:
     """Copy (selected) rows of a float matrix into a new matrix of ``dtype``."""
     _dev(x, rows)
@@ -293,7 +336,7 @@ PARTIAL_SHAPE = (-1, 4, 4)          # x resident in LDS, phases of 512 columns: 
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_pairs: bool = False,
-                block_shape=(0, 0, 0), out=None, ksplit: int = 1) -> torch.Tensor:
+                block_shape=(0, 0, 0), out=None, ksplit: int = 1, row_scale: "UnscaledRows | None" = None) -> torch.Tensor:
     """x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w [N, K]: the weight-streaming
     product of decode steps.  With ``silu_pairs`` the rows of w alternate gate and up rows and
     the result is silu(x.w[2j]) * (x.w[2j+1]), bfloat16 [M, N/2].  Output bfloat16 or float32.
@@ -302,7 +345,9 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     (-2, blocks, pieces) the one with blocks that stay and keep x in registers (at most 16 rows,
     inner size at most 256 * pieces).
     ``ksplit`` > 1 (that organisation, float32 output): the inner size is shared out to so many
-    blocks per row tile and the result is [ksplit, M, N], partial products to be added in order."""
+    blocks per row tile and the result is [ksplit, M, N], partial products to be added in order.
+    ``row_scale`` (blocks that stay only): x is ``row_scale.x``, un-normalised rows, and every output
+    row (of every partial product) is multiplied by its norm's scale."""
     _dev(x, w, out)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_skinny takes bfloat16")
     m = x.shape[0]
@@ -326,13 +371,19 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     _need(out.shape == shape and out.dtype == out_dtype and out.is_contiguous(),
           "out must be [M, N] (or [M, N/2], or [ksplit, M, N]) of the output type")
-    _check(
-        library.core().jv_gemm_skinny_bf16(
-            _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.stride(0)), c_longlong(n_out),
-            c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_pairs else 0),
-            c_int(block_shape[0]), c_int(block_shape[1]), c_int(block_shape[2]), c_int(ksplit), _stream()),
-        "gemm_skinny",
-    )
+    common = (_ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.stride(0)), c_longlong(n_out),
+              c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_pairs else 0),
+              c_int(block_shape[0]), c_int(block_shape[1]), c_int(block_shape[2]), c_int(ksplit))
+    if row_scale is not None:
+        _need(block_shape[0] == -2, "only the blocks that stay scale their output rows")
+        _need(row_scale.x is x and row_scale.ssq.is_cuda and row_scale.ssq.dtype == torch.float32
+              and row_scale.ssq.is_contiguous() and tuple(row_scale.ssq.shape) == (m, UNSCALED_MAX_SHARES)
+              and 1 <= row_scale.shares <= UNSCALED_MAX_SHARES, "row_scale does not belong to x")
+        _check(library.core().jv_gemm_skinny_scaled_bf16(*common, _ptr(row_scale.ssq), c_int(row_scale.shares),
+                                                         c_int(row_scale.width), c_float(row_scale.eps), _stream()),
+               "gemm_skinny")
+        return out
+    _check(library.core().jv_gemm_skinny_bf16(*common, _stream()), "gemm_skinny")
     return out
 
 
@@ -490,25 +541,40 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
     silu(x.w[2j]) * (x.w[2j+1]) of width N/2 (an epilogue of the streaming kernels, a kernel of
     its own after the library's product).
     """
+    scale = None
+    if isinstance(x, UnscaledRows):
+        scale, x = x, x.x
     if x.dtype == torch.float32:
         y = gemm_f32(x, w)
     else:
         _need(x.dtype == w.dtype, "x and w must have one type")
         plan = streaming_plan(x.shape[0], w.shape[0], w.shape[1], silu_pairs,
                               partial_ok and out_dtype in (None, torch.bfloat16), x.device, partial_max_width)
+        _need(scale is None or (plan is not None and plan[0][0] == -2),
+              "un-normalised rows need a product by the blocks that stay (ask linear_takes_unscaled_rows first)")
         if plan is not None:
             shape, parts = plan
             if shape == TILE64:
                 return gemm_tile64(x, w, torch.float32, ksplit=parts)
             if parts > 1:
-                return gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=parts)
-            return gemm_skinny(x, w, out_dtype or torch.bfloat16, silu_pairs=silu_pairs, block_shape=shape)
+                return gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=parts, row_scale=scale)
+            return gemm_skinny(x, w, out_dtype or torch.bfloat16, silu_pairs=silu_pairs, block_shape=shape,
+                               row_scale=scale)
         y = torch.mm(x, w.t())
     if silu_pairs:
         return silu_mul(y, interleaved=True)
     if out_dtype is not None and y.dtype != out_dtype:
         y = y.to(out_dtype)
     return y
+
+
+def linear_takes_unscaled_rows(n_rows: int, w: torch.Tensor, silu_pairs: bool = False, partial_ok: bool = False,
+                               partial_max_width: int | None = PARTIAL_SUM_MAX_WIDTH) -> bool:
+    """Whether ``linear`` with these arguments multiplies ``UnscaledRows`` (its plan is the blocks that stay)."""
+    if w.dtype != torch.bfloat16 or not unscaled_rows_possible(torch.bfloat16, n_rows, w.shape[1]):
+        return False
+    plan = streaming_plan(n_rows, w.shape[0], w.shape[1], silu_pairs, partial_ok, w.device, partial_max_width)
+    return plan is not None and plan[0] != TILE64 and plan[0][0] == -2
 
 
 # --------------------------------------------------------------------------- sampling

@@ -69,8 +69,18 @@ class GroupedQueryAttention:
         if self.position is not None:
             self.position.bind({}, dtype, self.w_o.device)
 
+    def takes_unscaled_rows(self, n_rows: int) -> bool:
+        """x goes into the qkv product and nowhere else: the norm before may leave its scale to that product."""
+        if self.position is None:
+            partial_ok = K.rope_takes_parts(self.dtype, self.d, False, 0, False)
+        elif hasattr(self.position, "rotary_dim") and hasattr(self.position, "interleaved"):
+            partial_ok = K.rope_takes_parts(self.dtype, self.d, self.position.interleaved, self.position.rotary_dim, True)
+        else:
+            return False        # an encoding that tells its rotation only step by step: the product's plan is not known here
+        return K.linear_takes_unscaled_rows(n_rows, self.w_qkv, partial_ok=partial_ok, partial_max_width=None)
+
     # ---- one step
-    def forward(self, x: torch.Tensor, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
+    def forward(self, x, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
         n = x.shape[0]
         cos_sin, rotary_dim, interleaved = (
             self.position.fused_arguments(ctx) if self.position is not None else (None, 0, False)

@@ -36,10 +36,17 @@ class PreNormBlock:
             part.bind({k[len(name) + 1:]: v for k, v in tensors.items() if k.startswith(name + ".")}, dtype)
 
     def forward(self, h, delta, mixer, feed_forward, ctx, mem):
-        x = self.mixer_norm.add_norm(h, delta)
+        # a part that says so (``takes_unscaled_rows(rows)``) may get ``K.UnscaledRows`` from the norm
+        n = h.shape[0]
+        x = self.mixer_norm.add_norm(h, delta, unscaled_ok=_takes_unscaled(mixer, n))
         a = mixer.forward(x, ctx, mem)
-        y = self.feed_forward_norm.add_norm(h, a)
+        y = self.feed_forward_norm.add_norm(h, a, unscaled_ok=_takes_unscaled(feed_forward, n))
         return feed_forward.forward(y, ctx)
+
+
+def _takes_unscaled(part, n_rows: int) -> bool:
+    ask = getattr(part, "takes_unscaled_rows", None)
+    return bool(ask is not None and ask(n_rows))
 
 
 register_part("block", "prenorm", PreNormBlock)

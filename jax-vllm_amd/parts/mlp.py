@@ -33,7 +33,11 @@ class GatedMLP:
         self.w_gate_up = torch.stack([g, u], dim=1).reshape(2 * g.shape[0], g.shape[1]).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
-    def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+    def takes_unscaled_rows(self, n_rows: int) -> bool:
+        """x goes into the gate/up product and nowhere else: the norm before may leave its scale to that product."""
+        return K.linear_takes_unscaled_rows(n_rows, self.w_gate_up, silu_pairs=True)
+
+    def forward(self, x, ctx=None) -> torch.Tensor:
         z = K.linear(x, self.w_gate_up, silu_pairs=True)    # gate and up rows alternate in the fused weight
         return K.linear(z, self.w_down, partial_ok=True)   # the next norm adds the partial products
 

@@ -821,6 +821,48 @@ def test_gemm_tile64_silu_epilogue_and_refusals():
         K().gemm_tile64(x, w, silu_pairs=True, ksplit=2, out_dtype=torch.float32)   # no activation of a partial sum
 
 
+@pytest.mark.parametrize("m,hidden,n_parts", [(8, 4096, 4), (1, 512, 2), (16, 5120, 3), (5, 8192, 1)])
+def test_residual_step_that_leaves_the_scale_to_the_product(m, hidden, n_parts):
+    """``add_parts_unscaled`` adds the partial products to the residual stream and hands on h * weight
+    with the shares of each row's sum of squares; a product by the blocks that stay multiplies its
+    output rows by the norm's scale.  Together they equal norm-then-product."""
+    kern = K()
+    h = randn(m, hidden, seed=70, scale=2.0)
+    parts = randn(n_parts, m, hidden, seed=71)
+    weight = 1 + 0.1 * randn(hidden, seed=72)
+    eps = 1e-5
+    total = parts[0]
+    for q in range(1, n_parts):
+        total = total + parts[q]
+    want_h = h + total
+    h2 = h.clone()
+    rows = kern.add_parts_unscaled(h2, parts, weight, eps)
+    torch.testing.assert_close(h2, want_h, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(rows.x.float(), (want_h * weight).to(torch.bfloat16).float(), rtol=0, atol=0)
+    assert rows.ssq.shape == (m, 16) and rows.shares == hidden // 512
+    torch.testing.assert_close(rows.ssq[:, :rows.shares].sum(-1), (want_h * want_h).sum(-1), rtol=1e-5, atol=1e-5)
+    # the product: qkv-like (partial products) and gate/up-like (activation as epilogue)
+    inv = torch.rsqrt((want_h.double() ** 2).mean(-1, keepdim=True) + eps)
+    xn = rows.x.double() * inv                      # what the reader multiplies, to the rounding of x
+    n = 1024
+    w = randn(n, hidden, dtype=torch.bfloat16, seed=73, scale=0.05)
+    assert kern.linear_takes_unscaled_rows(m, w, partial_ok=True) == (hidden != 512)     # no piece count covers 512 columns
+    if kern.linear_takes_unscaled_rows(m, w, partial_ok=True):
+        y = kern.linear(rows, w, partial_ok=True)
+        y = y.sum(0) if y.dim() == 3 else y.float()
+        torch.testing.assert_close(y.double(), xn @ w.double().T, rtol=2e-2, atol=2e-2)
+    wide = randn(2 * 16 * 4 * 256, hidden, dtype=torch.bfloat16, seed=74, scale=0.05)     # 1,024 row tiles: the wide plan
+    if kern.linear_takes_unscaled_rows(m, wide, silu_pairs=True):
+        z = kern.linear(rows, wide, silu_pairs=True)
+        full = xn @ wide.double().T
+        gate, up = full[:, 0::2], full[:, 1::2]
+        torch.testing.assert_close(z.double(), gate / (1 + torch.exp(-gate)) * up, rtol=3e-2, atol=3e-2)
+    # rows that were not made for this x are refused, and so is a plan that cannot scale
+    other = kern.UnscaledRows(rows.x.clone(), rows.ssq, hidden, eps)
+    with pytest.raises(kern.KernelArgumentError, match="does not belong"):
+        kern.gemm_skinny(rows.x, w, torch.float32, block_shape=(-2, 64, 4), ksplit=max(1, -(-hidden // 1024)), row_scale=other)
+
+
 def test_linear_takes_blocks_of_64_rows_for_a_long_inner_size():
     """17..64 rows against a narrow matrix with a long inner size (the feed-forward's second product):
     ``linear`` hands out partial products from ``gemm_tile64`` that ``add_rmsnorm`` adds; the same
