@@ -186,10 +186,11 @@ gemm_skinny_resident_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, 
   const int tid = threadIdx.x, nthreads = blockDim.x;
   const int wk = tid >> 6, lane = tid & 63, li = lane & 15, lc = lane >> 4;
   const int n = blockIdx.x * 16 + li;
-  const bool n_ok = n < N;
   const int kb = blockIdx.y * k_per;         // this block's columns are [kb, kb + K)
   const int K = K_all - kb < k_per ? K_all - kb : k_per;
-  const bf16_t* wrow = W + (long long)(n_ok ? n : 0) * K_all + kb + lc * 8;
+  // no load inside a branch: a row beyond N reads the last row (its outputs are never stored), a piece
+  // beyond the block's columns reads the row's last piece again, against zeros in x
+  const bf16_t* wrow = W + (long long)min(n, N - 1) * K_all + kb;
   x += kb;
   y += blockIdx.y * y_part;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -204,10 +205,7 @@ gemm_skinny_resident_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, 
     const int k0 = p * KP + wk * SL;
     bf16x8 a[NL];
 #pragma unroll
-    for (int i = 0; i < NL; ++i) {
-      const int k = k0 + i * 32 + lc * 8;
-      a[i] = (n_ok && k < K) ? *(const bf16x8*)(wrow + k0 + i * 32) : zero;
-    }
+    for (int i = 0; i < NL; ++i) a[i] = *(const bf16x8*)(wrow + min(k0 + i * 32 + lc * 8, K - 8));
     __syncthreads();  // zero fill (first phase) or the previous phase's reads are done
     for (int c = tid; c < xvecs; c += nthreads) {
       const int m = c / (KP / 8), kc = c - m * (KP / 8);
