@@ -509,7 +509,7 @@ __global__ void __launch_bounds__(256) PREFILL_OCCUPANCY attn_prefill_kernel(Att
 //     xor-ed with the line number: reads of 32 rows at one column and writes of whole rows are
 //     both conflict-free (measured).
 // Tiles are double-buffered in LDS: one barrier per 64 keys.  With pages of 16 keys and a head size
-// that is a power of two (PIPE) a wave also overlaps its own work: the scores of tile i + 1 are
+// that is a power of two (PAGES == 16) a wave also overlaps its own work: the scores of tile i + 1 are
 // multiplied while the probabilities of tile i are made (measured at 32 q heads over 8 kv heads of
 // 128: 2,048 tokens 58 against 63 us, 8,192 tokens 566 against 638, 512 tokens after 16,000: 306
 // against 383; the kernel then keeps the matrix unit busy 55..60 % of the time at the 1.9 GHz it
@@ -530,7 +530,7 @@ constexpr int PCS = BN * CPK / 256;        // 16-byte pieces of a K tile (and of
 constexpr bool KB_ADDS = (32 * CPK / 16) % 16 == 0;   // the second key block's chunks are the first's plus a constant
 __device__ __forceinline__ int swizzle(int q) { return q ^ ((q >> 4) & 15); }   // chunk index -> chunk position
 
-template <int PAGES, bool PIPE = false>
+template <int PAGES>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) attn_prefill32_kernel(AttnArgs p) {
   __shared__ __attribute__((aligned(16))) bf16_t Ks[2][BN * D];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[2][D * BN];
@@ -675,16 +675,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       int pi = (j0 >> 4) + (((4 * i + wave) * 64) / (2 * D));   // first key of the instruction, (4i + w) * 64 / CPK, over 16
       if (pi > last_page) pi = last_page;
       pg[i] = (unsigned)ctable[pi];
-    }
-  };
-  auto fetch_fast = [&](int b, const unsigned (&pg)[PCS]) {
-#pragma unroll
-    for (int i = 0; i < PCS; ++i) {
-      const unsigned long long base = (unsigned long long)pg[i] * page_stride;   // scalar
-      dma16(p.k_pages + base + (unsigned)k_off[i],
-              &Ks[b][(4 * i + wave) * 64 * 8]);
-      dma16(p.v_pages + base + (unsigned)v_off[i],
-              &Vs[b][(4 * i + wave) * 64 * 8]);
     }
   };
   auto fetch = [&](int j0, int b) {
@@ -859,7 +849,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     JV_PRIO(0);
   };
 
-  if constexpr (PIPE && FAST) {
+  if constexpr (FAST) {
     // ---- the same walk with a wave's products and its softmax overlapped: while the probabilities of tile i
     // are made (float units), the scores of tile i + 1 are already multiplied (matrix unit), and the first
     // products of O^T += V^T P^T start as soon as their 16 keys' probabilities exist.  K is therefore
@@ -1072,37 +1062,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       else tile_sm(sb, j0, Vs[1]);
     }
   } else {
-  unsigned pg[PCS];
-  if (FAST) {
-    pages_of(j_first, pg);
-    fetch_fast(0, pg);
-    if (next_tile(j_first) < kv_end) pages_of(next_tile(j_first), pg);
-  } else {
     fetch(j_first, 0);
-  }
-  arrived();
-  if (j_first + BN > kv_end) fix_tail(j_first, 0);
-  __syncthreads();
-  int b = 0;
-  for (int j0 = j_first; j0 < kv_end;) {
-    const int j_next = next_tile(j0);
-    const bool more = j_next < kv_end;
-    if (more) {                                     // in flight while this tile is multiplied; nobody reads that
-      if (FAST) {                                   // buffer: its tile was finished before the last barrier
-        fetch_fast(b ^ 1, pg);
-        const int j_after = next_tile(j_next);
-        if (j_after < kv_end) pages_of(j_after, pg);
-      } else {
-        fetch(j_next, b ^ 1);
-      }
-    }
-    if (wave_live && j0 < wave_kv_end && j0 + BN > wave_kv_begin) multiply(j0, b);
     arrived();
-    if (more && j_next + BN > kv_end) fix_tail(j_next, b ^ 1);   // own pieces only: no barrier needed before
+    if (j_first + BN > kv_end) fix_tail(j_first, 0);
     __syncthreads();
-    j0 = j_next;
-    b ^= 1;
-  }
+    int b = 0;
+    for (int j0 = j_first; j0 < kv_end;) {
+      const int j_next = next_tile(j0);
+      const bool more = j_next < kv_end;
+      if (more) fetch(j_next, b ^ 1);                 // in flight while this tile is multiplied; nobody reads that
+                                                      // buffer: its tile was finished before the last barrier
+      if (wave_live && j0 < wave_kv_end && j0 + BN > wave_kv_begin) multiply(j0, b);
+      arrived();
+      if (more && j_next + BN > kv_end) fix_tail(j_next, b ^ 1);   // own pieces only: no barrier needed before
+      __syncthreads();
+      j0 = j_next;
+      b ^= 1;
+    }
   }
 
   float l = l_lane + __shfl_xor(l_lane, 32, 64);
@@ -1436,7 +1412,7 @@ extern "C" int jv_attn_prefill(void* out, const void* q, long long q_row_stride,
   const int mode = (a.page_shift >= 3 && a.page_shift <= 6) ? 1 : (a.page_shift > 6 ? 2 : 0);
 #ifdef JV_PREFILL32
   constexpr bool pow2 = (D & (D - 1)) == 0;
-  void (*kernel)(AttnArgs) = (page_size == 16 && pow2) ? attn_prefill32_kernel<pow2 ? 16 : 1, pow2>
+  void (*kernel)(AttnArgs) = (page_size == 16 && pow2) ? attn_prefill32_kernel<pow2 ? 16 : 1>
                              : mode == 1 ? attn_prefill32_kernel<1>
                              : mode == 2 ? attn_prefill32_kernel<2> : attn_prefill32_kernel<0>;
 #else
