@@ -42,4 +42,17 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// Gate activations of a gated feed-forward, y = act(gate) * up, in float.  The ids are part of the
+// exported interface (the Python side names them).
+#define JV_ACT_SILU 1        // gate / (1 + exp(-gate))
+#define JV_ACT_GELU_TANH 2   // 0.5 gate (1 + tanh(sqrt(2/pi) (gate + 0.044715 gate^3)))
+__host__ __device__ __forceinline__ bool jv_act_known(int act) { return act == JV_ACT_SILU || act == JV_ACT_GELU_TANH; }
+__device__ __forceinline__ float jv_gated(int act, float gate, float up) {
+  if (act == JV_ACT_GELU_TANH) {
+    const float inner = 0.7978845608028654f * (gate + 0.044715f * gate * gate * gate);
+    return 0.5f * gate * (1.f + tanhf(inner)) * up;
+  }
+  return gate / (1.f + expf(-gate)) * up;
+}
+
 #define JV_LAUNCH_CHECK() ((int)hipGetLastError())

@@ -281,13 +281,13 @@ __global__ void rmsnorm_kernel(T* __restrict__ out, const T* __restrict__ x,
   for (int c = lane; c < n; c += JV_WAVE) o[c] = from_f32<T>(to_f32(xr[c]) * inv * w[c]);
 }
 
-// ---------------------------------------------------------------- SiLU-mul
-// out[t, j] = silu(gate) * up, silu(x) = x / (1 + exp(-x)), in float.  Two layouts of gu[t, 2*inter]:
+// ---------------------------------------------------------------- gate activation times up
+// out[t, j] = act(gate) * up in float, act one of JV_ACT_*.  Two layouts of gu[t, 2*inter]:
 // halves (gate = gu[t, j], up = gu[t, inter + j]) or interleaved (gate = gu[t, 2j], up = gu[t, 2j+1]).
-// Interleaved layout (gate and up alternate along the row): out[t, j] = silu(gu[t, 2j]) * gu[t, 2j+1];
+// Interleaved layout (gate and up alternate along the row): out[t, j] = act(gu[t, 2j]) * gu[t, 2j+1];
 // each thread takes four outputs (8 inputs, 16 bytes of bfloat16) when inter % 4 == 0.
-template <typename T>
-__global__ void silu_mul_pairs_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
+template <typename T, int ACT>
+__global__ void gated_mul_pairs_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
   const long long t = blockIdx.y;
   const int j = (blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (j >= inter) return;
@@ -296,19 +296,17 @@ __global__ void silu_mul_pairs_kernel(T* __restrict__ out, const T* __restrict__
   if ((inter & 3) == 0) {
     float v[8];
     load8<T>(gp, v);
-    store4<T>(op, float4{v[0] / (1.f + expf(-v[0])) * v[1], v[2] / (1.f + expf(-v[2])) * v[3],
-                         v[4] / (1.f + expf(-v[4])) * v[5], v[6] / (1.f + expf(-v[6])) * v[7]});
+    store4<T>(op, float4{jv_gated(ACT, v[0], v[1]), jv_gated(ACT, v[2], v[3]), jv_gated(ACT, v[4], v[5]),
+                         jv_gated(ACT, v[6], v[7])});
   } else {
-    for (int e = 0; e < 4 && j + e < inter; ++e) {
-      const float g = to_f32(gp[2 * e]), u = to_f32(gp[2 * e + 1]);
-      op[e] = from_f32<T>(g / (1.f + expf(-g)) * u);
-    }
+    for (int e = 0; e < 4 && j + e < inter; ++e)
+      op[e] = from_f32<T>(jv_gated(ACT, to_f32(gp[2 * e]), to_f32(gp[2 * e + 1])));
   }
 }
 
 // grid (column blocks, tokens); each thread takes 4 neighbouring columns when inter % 4 == 0.
-template <typename T, int VEC>
-__global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
+template <typename T, int VEC, int ACT>
+__global__ void gated_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, int inter) {
   const long long t = blockIdx.y;
   const int j = (blockIdx.x * blockDim.x + threadIdx.x) * VEC;
   if (j >= inter) return;
@@ -316,12 +314,24 @@ __global__ void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ gu, i
   T* op = out + t * inter + j;
   if (VEC == 4) {
     const float4 g = load4<T>(gp), u = load4<T>(gp + inter);
-    store4<T>(op, float4{g.x / (1.f + expf(-g.x)) * u.x, g.y / (1.f + expf(-g.y)) * u.y,
-                         g.z / (1.f + expf(-g.z)) * u.z, g.w / (1.f + expf(-g.w)) * u.w});
+    store4<T>(op, float4{jv_gated(ACT, g.x, u.x), jv_gated(ACT, g.y, u.y), jv_gated(ACT, g.z, u.z),
+                         jv_gated(ACT, g.w, u.w)});
   } else {
-    const float g = to_f32(gp[0]), u = to_f32(gp[inter]);
-    op[0] = from_f32<T>(g / (1.f + expf(-g)) * u);
+    op[0] = from_f32<T>(jv_gated(ACT, to_f32(gp[0]), to_f32(gp[inter])));
   }
+}
+
+template <typename T, int ACT>
+static void launch_gated_mul(T* o, const T* g, unsigned ny, int inter, int interleaved, hipStream_t stream) {
+  if (interleaved)
+    hipLaunchKernelGGL((gated_mul_pairs_kernel<T, ACT>), dim3(((inter + 3) / 4 + 255) / 256, ny), dim3(256), 0, stream,
+                       o, g, inter);
+  else if (inter % 4 == 0)
+    hipLaunchKernelGGL((gated_mul_kernel<T, 4, ACT>), dim3((inter / 4 + 255) / 256, ny), dim3(256), 0, stream, o, g,
+                       inter);
+  else
+    hipLaunchKernelGGL((gated_mul_kernel<T, 1, ACT>), dim3((inter + 255) / 256, ny), dim3(256), 0, stream, o, g,
+                       inter);
 }
 
 // ---------------------------------------------------------------- float -> T copy of selected rows
@@ -404,23 +414,18 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
                        n, eps);                                                                     \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \
-  extern "C" int jv_silu_mul_##SUF(void* out, const void* gu, long long n_tokens, int inter,        \
-                                   int interleaved, void* stream) {                                 \
+  extern "C" int jv_gated_mul_##SUF(void* out, const void* gu, long long n_tokens, int inter,       \
+                                    int interleaved, int act, void* stream) {                      \
     if (n_tokens <= 0 || inter <= 0) return 0;                                                      \
+    if (!jv_act_known(act)) return (int)hipErrorInvalidValue;                                       \
     for (long long t0 = 0; t0 < n_tokens; t0 += 65535) { /* grid.y limit */                         \
       const unsigned ny = (unsigned)(n_tokens - t0 < 65535 ? n_tokens - t0 : 65535);                \
       T* o = (T*)out + t0 * inter;                                                                  \
       const T* g = (const T*)gu + t0 * 2 * inter;                                                   \
-      if (interleaved) {                                                                            \
-        hipLaunchKernelGGL((silu_mul_pairs_kernel<T>), dim3(((inter + 3) / 4 + 255) / 256, ny),     \
-                           dim3(256), 0, (hipStream_t)stream, o, g, inter);                         \
-      } else if (inter % 4 == 0) {                                                                         \
-        hipLaunchKernelGGL((silu_mul_kernel<T, 4>), dim3((inter / 4 + 255) / 256, ny), dim3(256),   \
-                           0, (hipStream_t)stream, o, g, inter);                                    \
-      } else {                                                                                      \
-        hipLaunchKernelGGL((silu_mul_kernel<T, 1>), dim3((inter + 255) / 256, ny), dim3(256), 0,    \
-                           (hipStream_t)stream, o, g, inter);                                       \
-      }                                                                                             \
+      if (act == JV_ACT_GELU_TANH)                                                                  \
+        launch_gated_mul<T, JV_ACT_GELU_TANH>(o, g, ny, inter, interleaved, (hipStream_t)stream);   \
+      else                                                                                          \
+        launch_gated_mul<T, JV_ACT_SILU>(o, g, ny, inter, interleaved, (hipStream_t)stream);        \
     }                                                                                               \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \

@@ -14,7 +14,7 @@
 // order, so a result does not depend on M, on the grid or on timing.
 //
 // Optional epilogue for the feed-forward's first product: when the rows of W alternate gate and
-// up rows, y[m, j] = silu(x.W[2j]) * (x.W[2j+1]) straight from the float accumulators (a lane
+// up rows, y[m, j] = act(x.W[2j]) * (x.W[2j+1]) straight from the float accumulators (a lane
 // holds both numbers of a pair), which saves the activation kernel and its round trip.
 #include "common.h"
 
@@ -28,7 +28,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 template <int MT, int NKS, typename OutT, bool PAIRS>
 __global__ void __launch_bounds__(MT == 1 ? 1024 : 512)
 gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
-                   int M, int N, int K, long long ldx, long long ldy, int WR, int WK) {
+                   int M, int N, int K, long long ldx, long long ldy, int WR, int WK, int act) {
   constexpr int STEP = NKS * 32;
   constexpr int ROWS = MT * 16;
   constexpr int XP = 2 * MT;                 // x pieces a thread keeps in flight
@@ -150,11 +150,11 @@ gemm_skinny_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
     const int nb = (blockIdx.x * WR + wr) * 16 + lc * 4;
     if (m < M) {
       if (PAIRS) {
-        // rows of W alternate gate, up: column pair (2j, 2j+1) -> y[m, j] = silu(gate) * up
+        // rows of W alternate gate, up: column pair (2j, 2j+1) -> y[m, j] = act(gate) * up
 #pragma unroll
         for (int e = 0; e < 4; e += 2)
           if (nb + e + 1 < N)
-            y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(s[e] / (1.f + expf(-s[e])) * s[e + 1]);
+            y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(jv_gated(act, s[e], s[e + 1]));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -288,7 +288,7 @@ static size_t skinny_shmem(int MT, int NKS, int WR, int WK) {
 
 template <int MT, int NKS, typename OutT, bool PAIRS>
 static int launch_skinny(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                         long long ldy, int WR, int WK, hipStream_t stream) {
+                         long long ldy, int WR, int WK, int act, hipStream_t stream) {
   const size_t shmem = skinny_shmem(MT, NKS, WR, WK);
   if (shmem > 64 * 1024) {
     static bool raised = false;  // per instantiation
@@ -301,29 +301,29 @@ static int launch_skinny(void* y, const void* x, const void* W, int M, int N, in
   }
   const int blocks = (N + 16 * WR - 1) / (16 * WR);
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, NKS, OutT, PAIRS>), dim3(blocks), dim3(WR * WK * 64), shmem,
-                     stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, WR, WK);
+                     stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, WR, WK, act);
   return JV_LAUNCH_CHECK();
 }
 
 template <int NKS, typename OutT, bool PAIRS>
 static int dispatch_mt(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                       long long ldy, int WR, int WK, hipStream_t s) {
+                       long long ldy, int WR, int WK, int act, hipStream_t s) {
   switch ((M + 15) / 16) {
-    case 1: return launch_skinny<1, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 2: return launch_skinny<2, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 3: return launch_skinny<3, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 4: return launch_skinny<4, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 1: return launch_skinny<1, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, act, s);
+    case 2: return launch_skinny<2, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, act, s);
+    case 3: return launch_skinny<3, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, act, s);
+    case 4: return launch_skinny<4, NKS, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, act, s);
   }
   return (int)hipErrorInvalidValue;
 }
 
 template <typename OutT, bool PAIRS>
 static int dispatch_nks(int nks, void* y, const void* x, const void* W, int M, int N, int K,
-                        long long ldx, long long ldy, int WR, int WK, hipStream_t s) {
+                        long long ldx, long long ldy, int WR, int WK, int act, hipStream_t s) {
   switch (nks) {
-    case 2: return dispatch_mt<2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 4: return dispatch_mt<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
-    case 8: return dispatch_mt<8, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, s);
+    case 2: return dispatch_mt<2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, act, s);
+    case 4: return dispatch_mt<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, act, s);
+    case 8: return dispatch_mt<8, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, WR, WK, act, s);
   }
   return (int)hipErrorInvalidValue;
 }
@@ -343,6 +343,7 @@ struct RowScale {
   const float* ssq;
   int shares;       // at most 16
   float inv_width, eps;
+  int act;          // PAIRS: the gate's activation (JV_ACT_*)
 };
 
 // No load of the loop sits inside a branch (the compiler would wrap each in a branch of its own, and wait at
@@ -426,7 +427,7 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
 #pragma unroll
           for (int e = 0; e < 4; e += 2)
             if (nb + e + 1 < N)
-              y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(s[e] / (1.f + expf(-s[e])) * s[e + 1]);
+              y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(jv_gated(rs.act, s[e], s[e + 1]));
         } else {
 #pragma unroll
           for (int e = 0; e < 4; ++e)
@@ -536,25 +537,26 @@ static void skinny_config(int M, int N, int K, int* wr, int* wk, int* nks) {
 }
 
 // out_f32: 0 -> y is bf16, 1 -> y is float.  x is [M, K] with row stride ldx.
-// silu_pairs: 1 -> the rows of W alternate gate and up rows and y[m, j] =
-//      silu(x.W[2j]) * (x.W[2j+1]) is bf16 [M, N/2] (the feed-forward's first product with its
+// gate_act: JV_ACT_* (not 0) -> the rows of W alternate gate and up rows and y[m, j] =
+//      act(x.W[2j]) * (x.W[2j+1]) is bf16 [M, N/2] (a gated feed-forward's first product with its
 //      activation as epilogue).
 // wr, wk, nks: block shape (row tiles, K slices, MFMA steps per iteration); 0 picks them.
-// wr == -1 selects the resident-x organisation (M <= 16, no silu): wk waves, nks in {2, 4, 8, 16}
+// wr == -1 selects the resident-x organisation (M <= 16, no activation): wk waves, nks in {2, 4, 8, 16}
 // weight pieces per wave and phase.
 // ksplit > 1 (resident-x organisation or blocks that stay, float output only): K is shared out to ksplit blocks per
 // row tile and y is [ksplit][M][ldy], partial products that the reader adds in that order.
 static int gemm_skinny_entry(void* y, const void* x, const void* W, int M, int N, int K, long long ldx, long long ldy,
-                             int out_f32, int silu_pairs, int wr, int wk, int nks, int ksplit, RowScale rs,
+                             int out_f32, int gate_act, int wr, int wk, int nks, int ksplit, RowScale rs,
                              void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (rs.ssq && (wr != -2 || rs.shares < 1 || rs.shares > 16)) return (int)hipErrorInvalidValue;   // only the staying blocks scale rows
   if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
-  if (silu_pairs && (out_f32 || N % 2 != 0 || wr == -1)) return (int)hipErrorInvalidValue;
+  if (gate_act && (!jv_act_known(gate_act) || out_f32 || N % 2 != 0 || wr == -1)) return (int)hipErrorInvalidValue;
+  rs.act = gate_act;
   if (ksplit < 1 || (ksplit > 1 && ((wr != -1 && wr != -2) || !out_f32))) return (int)hipErrorInvalidValue;
   if (wr == -2) {   // blocks that stay: wk = number of blocks, nks = weight pieces per wave
     hipStream_t s = (hipStream_t)stream;
-    if (silu_pairs) return dispatch_persistent<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, rs, s);
+    if (gate_act) return dispatch_persistent<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, rs, s);
     return out_f32 ? dispatch_persistent<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, rs, s)
                    : dispatch_persistent<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, rs, s);
   }
@@ -564,7 +566,7 @@ static int gemm_skinny_entry(void* y, const void* x, const void* W, int M, int N
     return out_f32 ? dispatch_resident<float>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s)
                    : dispatch_resident<bf16_t>(nks, y, x, W, M, N, K, ldx, ldy, wk, ksplit, s);
   }
-  if (wr == 0 && wk == 0 && nks == 0 && M <= 2 && !silu_pairs && K >= 2048 && K <= 4096 && N >= 8192) {
+  if (wr == 0 && wk == 0 && nks == 0 && M <= 2 && !gate_act && K >= 2048 && K <= 4096 && N >= 8192) {
     // one or two rows against a wide matrix: the resident-x organisation measured ~10 % faster
     hipStream_t s = (hipStream_t)stream;
     return out_f32 ? dispatch_resident<float>(16, y, x, W, M, N, K, ldx, ldy, 8, 1, s)
@@ -579,25 +581,25 @@ static int gemm_skinny_entry(void* y, const void* x, const void* W, int M, int N
   if (wr * wk > (MT == 1 ? 16 : 8) || (nks != 2 && nks != 4 && nks != 8)) return (int)hipErrorInvalidValue;
   if (skinny_shmem(MT, nks, wr, wk) > 160 * 1024) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
-  if (silu_pairs) return dispatch_nks<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
-  if (out_f32) return dispatch_nks<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
-  return dispatch_nks<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, s);
+  if (gate_act) return dispatch_nks<bf16_t, true>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, gate_act, s);
+  if (out_f32) return dispatch_nks<float, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, 0, s);
+  return dispatch_nks<bf16_t, false>(nks, y, x, W, M, N, K, ldx, ldy, wr, wk, 0, s);
 }
 
 extern "C" int jv_gemm_skinny_bf16(void* y, const void* x, const void* W, int M, int N, int K,
-                                   long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
+                                   long long ldx, long long ldy, int out_f32, int gate_act, int wr,
                                    int wk, int nks, int ksplit, void* stream) {
-  return gemm_skinny_entry(y, x, W, M, N, K, ldx, ldy, out_f32, silu_pairs, wr, wk, nks, ksplit,
-                           RowScale{nullptr, 0, 0.f, 0.f}, stream);
+  return gemm_skinny_entry(y, x, W, M, N, K, ldx, ldy, out_f32, gate_act, wr, wk, nks, ksplit,
+                           RowScale{nullptr, 0, 0.f, 0.f, 0}, stream);
 }
 
 // The same for rows of x that add_parts_unscaled left un-normalised (blocks that stay only, wr == -2):
 // output row m is multiplied by rsqrt(sum_{j < shares} ssq[m * 16 + j] / width + eps).
 extern "C" int jv_gemm_skinny_scaled_bf16(void* y, const void* x, const void* W, int M, int N, int K,
-                                          long long ldx, long long ldy, int out_f32, int silu_pairs, int wr,
+                                          long long ldx, long long ldy, int out_f32, int gate_act, int wr,
                                           int wk, int nks, int ksplit, const float* ssq, int shares, int width,
                                           float eps, void* stream) {
   if (!ssq || width <= 0) return (int)hipErrorInvalidValue;
-  return gemm_skinny_entry(y, x, W, M, N, K, ldx, ldy, out_f32, silu_pairs, wr, wk, nks, ksplit,
-                           RowScale{ssq, shares, 1.f / (float)width, eps}, stream);
+  return gemm_skinny_entry(y, x, W, M, N, K, ldx, ldy, out_f32, gate_act, wr, wk, nks, ksplit,
+                           RowScale{ssq, shares, 1.f / (float)width, eps, 0}, stream);
 }

@@ -26,7 +26,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 template <int MT, typename OutT, bool PAIRS>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))   // one block a compute unit, 256 registers a lane
 gemm_tile64_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
-                   int M, int N, int K, long long ldx, long long ldy, int k_per) {
+                   int M, int N, int K, long long ldx, long long ldy, int k_per, int act) {
   constexpr int ROWS = MT * 16;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   bf16_t (*xs)[ROWS * T64_XS] = (bf16_t (*)[ROWS * T64_XS])smem;   // [2][ROWS][T64_XS]
@@ -132,7 +132,7 @@ gemm_tile64_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
 #pragma unroll
         for (int e = 0; e < 4; e += 2)
           if (nb + e + 1 < N)
-            y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(s[e] / (1.f + expf(-s[e])) * s[e + 1]);
+            y[(long long)m * ldy + (nb + e) / 2] = from_f32<OutT>(jv_gated(act, s[e], s[e + 1]));
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
@@ -144,7 +144,7 @@ gemm_tile64_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf1
 
 template <int MT, typename OutT, bool PAIRS>
 static int launch_tile64(void* y, const void* x, const void* W, int M, int N, int K, long long ldx, long long ldy,
-                         int ksplit, hipStream_t stream) {
+                         int ksplit, int act, hipStream_t stream) {
   // columns per group: a whole number of chunks, every group with at least one column
   const int chunks = (K + T64_KC - 1) / T64_KC;
   const int k_per = ((chunks + ksplit - 1) / ksplit) * T64_KC;
@@ -160,36 +160,36 @@ static int launch_tile64(void* y, const void* x, const void* W, int M, int N, in
     }
   }
   hipLaunchKernelGGL((gemm_tile64_kernel<MT, OutT, PAIRS>), dim3((N + 63) / 64, ksplit), dim3(512), shmem, stream,
-                     (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, k_per);
+                     (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, k_per, act);
   return JV_LAUNCH_CHECK();
 }
 
 template <typename OutT, bool PAIRS>
 static int dispatch_tile64(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                           long long ldy, int ksplit, hipStream_t s) {
+                           long long ldy, int ksplit, int act, hipStream_t s) {
   switch ((M + 15) / 16) {
-    case 1: return launch_tile64<1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, s);
-    case 2: return launch_tile64<2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, s);
-    case 3: return launch_tile64<3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, s);
-    case 4: return launch_tile64<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, s);
+    case 1: return launch_tile64<1, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, act, s);
+    case 2: return launch_tile64<2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, act, s);
+    case 3: return launch_tile64<3, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, act, s);
+    case 4: return launch_tile64<4, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, ksplit, act, s);
   }
   return (int)hipErrorInvalidValue;
 }
 
 // out_f32: 0 -> y is bf16, 1 -> y is float.  x is [M, K] with row stride ldx, M <= 64.
-// silu_pairs: 1 -> the rows of W alternate gate and up rows and y[m, j] =
-//      silu(x.W[2j]) * (x.W[2j+1]) is bf16 [M, N/2].
-// ksplit > 1 (float output, no silu): K is shared out to ksplit blocks per tile of 64 rows of W
+// gate_act: JV_ACT_* (not 0) -> the rows of W alternate gate and up rows and y[m, j] =
+//      act(x.W[2j]) * (x.W[2j+1]) is bf16 [M, N/2].
+// ksplit > 1 (float output, no activation): K is shared out to ksplit blocks per tile of 64 rows of W
 // and y is [ksplit][M][ldy], partial products that the reader adds in that order; refused when
 // a group would be left without columns.
 extern "C" int jv_gemm_tile64_bf16(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
-                                   long long ldy, int out_f32, int silu_pairs, int ksplit, void* stream) {
+                                   long long ldy, int out_f32, int gate_act, int ksplit, void* stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % 8 != 0 || ldx % 8 != 0) return (int)hipErrorInvalidValue;
-  if (silu_pairs && (out_f32 || N % 2 != 0 || ksplit != 1)) return (int)hipErrorInvalidValue;
+  if (gate_act && (!jv_act_known(gate_act) || out_f32 || N % 2 != 0 || ksplit != 1)) return (int)hipErrorInvalidValue;
   if (ksplit < 1 || ksplit > 65535 || (ksplit > 1 && !out_f32)) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
-  if (silu_pairs) return dispatch_tile64<bf16_t, true>(y, x, W, M, N, K, ldx, ldy, ksplit, s);
-  return out_f32 ? dispatch_tile64<float, false>(y, x, W, M, N, K, ldx, ldy, ksplit, s)
-                 : dispatch_tile64<bf16_t, false>(y, x, W, M, N, K, ldx, ldy, ksplit, s);
+  if (gate_act) return dispatch_tile64<bf16_t, true>(y, x, W, M, N, K, ldx, ldy, ksplit, gate_act, s);
+  return out_f32 ? dispatch_tile64<float, false>(y, x, W, M, N, K, ldx, ldy, ksplit, 0, s)
+                 : dispatch_tile64<bf16_t, false>(y, x, W, M, N, K, ldx, ldy, ksplit, 0, s);
 }

@@ -122,7 +122,8 @@ def build_spec(cfg: Qwen3Config) -> ModelSpec:
             "position": PartSpec("rotary", {"head_dim": cfg.head_dim, "theta": cfg.rope_theta}),
         },
     )
-    ffn = PartSpec("gated_mlp", {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size})
+    ffn = PartSpec("gated_mlp", {"hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size,
+                                 "activation": "silu"})
     block = PartSpec("prenorm", {"norm": norm})
     layers = [
         LayerSpec(prefix=f"model.layers.{i}.", mixer=mixer, feed_forward=ffn, block=block,

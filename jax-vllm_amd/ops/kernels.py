@@ -189,9 +189,18 @@ def cast_rows(x: torch.Tensor, dtype: torch.dtype, rows=None) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- activation
-def silu_mul(gate_up: torch.Tensor, out=None, interleaved: bool = False) -> torch.Tensor:
-    """out[t, j] = silu(gate) * up for gate_up of width 2 I: gate = gate_up[t, j], up =
-    gate_up[t, I + j], or with ``interleaved`` gate = gate_up[t, 2j], up = gate_up[t, 2j + 1]."""
+GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}      # the kernels' ids of act in y = act(gate) * up
+
+
+def _gate_act_id(name) -> int:
+    _need(name in GATE_ACTIVATIONS, f"no kernel for the gate activation {name!r}: there are {sorted(GATE_ACTIVATIONS)}")
+    return GATE_ACTIVATIONS[name]
+
+
+def gated_mul(gate_up: torch.Tensor, out=None, interleaved: bool = False, activation: str = "silu") -> torch.Tensor:
+    """out[t, j] = act(gate) * up for gate_up of width 2 I: gate = gate_up[t, j], up =
+    gate_up[t, I + j], or with ``interleaved`` gate = gate_up[t, 2j], up = gate_up[t, 2j + 1];
+    ``activation`` is one of ``GATE_ACTIVATIONS``, computed in float."""
     _dev(gate_up)
     n, two_i = gate_up.shape
     _need(two_i % 2 == 0, "gate_up must have an even width")
@@ -200,9 +209,9 @@ def silu_mul(gate_up: torch.Tensor, out=None, interleaved: bool = False) -> torc
         out = torch.empty((n, inter), dtype=gate_up.dtype, device=gate_up.device)
     _dev(out)
     _need(out.shape == (n, inter) and out.dtype == gate_up.dtype, "out must be [tokens, I] of gate_up's type")
-    fn = getattr(library.core(), f"jv_silu_mul_{_suffix(gate_up.dtype)}")
-    _check(fn(_ptr(out), _ptr(gate_up), c_longlong(n), c_int(inter), c_int(1 if interleaved else 0), _stream()),
-           "silu_mul")
+    fn = getattr(library.core(), f"jv_gated_mul_{_suffix(gate_up.dtype)}")
+    _check(fn(_ptr(out), _ptr(gate_up), c_longlong(n), c_int(inter), c_int(1 if interleaved else 0),
+              c_int(_gate_act_id(activation)), _stream()), "gated_mul")
     return out
 
 
@@ -335,11 +344,11 @@ PARTIAL_BLOCKS = 1024               # a streaming product wants about this many 
 PARTIAL_SHAPE = (-1, 4, 4)          # x resident in LDS, phases of 512 columns: for inner sizes the staying blocks do not cover
 
 
-def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_pairs: bool = False,
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, gate_pairs: "str | None" = None,
                 block_shape=(0, 0, 0), out=None, ksplit: int = 1, row_scale: "UnscaledRows | None" = None) -> torch.Tensor:
     """x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w [N, K]: the weight-streaming
-    product of decode steps.  With ``silu_pairs`` the rows of w alternate gate and up rows and
-    the result is silu(x.w[2j]) * (x.w[2j+1]), bfloat16 [M, N/2].  Output bfloat16 or float32.
+    product of decode steps.  With ``gate_pairs`` (one of ``GATE_ACTIVATIONS``) the rows of w alternate gate
+    and up rows and the result is act(x.w[2j]) * (x.w[2j+1]), bfloat16 [M, N/2].  Output bfloat16 or float32.
     ``block_shape``: (row tiles, K slices, MFMA steps per iteration) of a block, zeros: chosen
     from the shape; (-1, waves, pieces) selects the organisation with x resident in LDS;
     (-2, blocks, pieces) the one with blocks that stay and keep x in registers (at most 16 rows,
@@ -360,19 +369,19 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
                                    and 256 * block_shape[2] * (ksplit - 1) < k <= 256 * block_shape[2] * ksplit),
           "the organisation with blocks that stay takes at most 16 rows (32 with at most 8 pieces) and an inner "
           "size of ksplit * 256 * pieces at most")
-    _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
-          "the silu epilogue writes bfloat16, needs an even number of rows of w and the chunked organisation")
+    _need(not gate_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
+          "the activation epilogue writes bfloat16, needs an even number of rows of w and the chunked organisation")
     _need(ksplit >= 1 and (ksplit == 1 or (block_shape[0] in (-1, -2) and out_dtype == torch.float32
                                            and (m <= 16 or block_shape[0] == -2))),
           "sharing the inner size out needs x resident (at most 16 rows) or blocks that stay, and float32 output")
-    n_out = n // 2 if silu_pairs else n
+    n_out = n // 2 if gate_pairs else n
     shape = (m, n_out) if ksplit == 1 else (ksplit, m, n_out)
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     _need(out.shape == shape and out.dtype == out_dtype and out.is_contiguous(),
           "out must be [M, N] (or [M, N/2], or [ksplit, M, N]) of the output type")
     common = (_ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.stride(0)), c_longlong(n_out),
-              c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_pairs else 0),
+              c_int(1 if out_dtype == torch.float32 else 0), c_int(_gate_act_id(gate_pairs) if gate_pairs else 0),
               c_int(block_shape[0]), c_int(block_shape[1]), c_int(block_shape[2]), c_int(ksplit))
     if row_scale is not None:
         _need(block_shape[0] == -2, "only the blocks that stay scale their output rows")
@@ -387,12 +396,12 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     return out
 
 
-def gemm_tile64(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu_pairs: bool = False,
+def gemm_tile64(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, gate_pairs: "str | None" = None,
                 ksplit: int = 1, out=None) -> torch.Tensor:
     """x @ w.T for at most 64 rows of bfloat16 x against bfloat16 w [N, K] with blocks that take 64
     rows of w against all rows of x: the weight-streaming product of decode steps with 17..64
-    requests where the library is slow (narrow outputs over a long inner size).  ``silu_pairs`` and ``ksplit`` as in ``gemm_skinny``:
-    silu(x.w[2j]) * (x.w[2j+1]) as bfloat16 [M, N/2], or float32 partial products [ksplit, M, N] to
+    requests where the library is slow (narrow outputs over a long inner size).  ``gate_pairs`` and ``ksplit`` as in ``gemm_skinny``:
+    act(x.w[2j]) * (x.w[2j+1]) as bfloat16 [M, N/2], or float32 partial products [ksplit, M, N] to
     be added in order (every group needs at least one round of 256 columns)."""
     _dev(x, w, out)
     _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16, "gemm_tile64 takes bfloat16")
@@ -404,12 +413,12 @@ def gemm_tile64(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
           "the inner size and the row stride must be multiples of 8")
     _need(w.is_contiguous(), "w must be contiguous")
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
-    _need(not silu_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and ksplit == 1),
-          "the silu epilogue writes bfloat16, needs an even number of rows of w and an inner size in one piece")
+    _need(not gate_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and ksplit == 1),
+          "the activation epilogue writes bfloat16, needs an even number of rows of w and an inner size in one piece")
     rounds = -(-k // 256)
     _need(ksplit >= 1 and (ksplit == 1 or (out_dtype == torch.float32 and -(-rounds // ksplit) * (ksplit - 1) < rounds)),
           "sharing the inner size out needs float32 output and a round of 256 columns for every group")
-    n_out = n // 2 if silu_pairs else n
+    n_out = n // 2 if gate_pairs else n
     shape = (m, n_out) if ksplit == 1 else (ksplit, m, n_out)
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
@@ -418,7 +427,7 @@ def gemm_tile64(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, silu
     _check(
         library.core().jv_gemm_tile64_bf16(
             _ptr(out), _ptr(x), _ptr(w), c_int(m), c_int(n), c_int(k), c_longlong(x.stride(0)), c_longlong(n_out),
-            c_int(1 if out_dtype == torch.float32 else 0), c_int(1 if silu_pairs else 0), c_int(ksplit), _stream()),
+            c_int(1 if out_dtype == torch.float32 else 0), c_int(_gate_act_id(gate_pairs) if gate_pairs else 0), c_int(ksplit), _stream()),
         "gemm_tile64",
     )
     return out
@@ -459,7 +468,7 @@ TILE64_MIN_SHARE = 3072             # columns a block of gemm_tile64 needs to pa
 LIBRARY_MAX_INNER = 12288           # beyond this inner size the library's choice for few rows collapses
 
 
-def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok: bool = False, device=None,
+def streaming_plan(m: int, n: int, k: int, gate_pairs: bool = False, partial_ok: bool = False, device=None,
                    partial_max_width: int | None = PARTIAL_SUM_MAX_WIDTH):
     """How ``linear`` runs a bfloat16 product at few rows: (block_shape, ksplit) for ``gemm_skinny``
     (``TILE64`` as block shape: for ``gemm_tile64``), or None for the library.  All thresholds are
@@ -492,7 +501,7 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     if k % 8:
         return None
     cus = compute_units(device) if device is not None else 256
-    narrow = partial_ok and not silu_pairs and n % 4 == 0 and (partial_max_width is None or n <= partial_max_width)
+    narrow = partial_ok and not gate_pairs and n % 4 == 0 and (partial_max_width is None or n <= partial_max_width)
     if m > SKINNY_AUTO_ROWS:
         if narrow and m <= SKINNY_MAX_ROWS:
             parts = _fit_parts(-(-k // 256), min(4, cus // -(-n // 64)))
@@ -526,7 +535,7 @@ def streaming_plan(m: int, n: int, k: int, silu_pairs: bool = False, partial_ok:
     return (0, 0, 0), 1
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = False, silu_pairs: bool = False,
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = False, gate_pairs: "str | None" = None,
            partial_max_width: int | None = PARTIAL_SUM_MAX_WIDTH):
     """x @ w.T for w stored [out, in].
 
@@ -537,9 +546,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
     With ``partial_ok`` the caller takes a float32 stack [parts, M, N] of partial products as well
     (to be added in order, as ``add_rmsnorm`` does); it is returned for narrow matrices at up to 64 rows
     (``partial_max_width``: the widest row whose parts the caller's reader adds; None: any).
-    With ``silu_pairs`` the rows of w alternate gate and up rows and the result is
-    silu(x.w[2j]) * (x.w[2j+1]) of width N/2 (an epilogue of the streaming kernels, a kernel of
-    its own after the library's product).
+    With ``gate_pairs`` (one of ``GATE_ACTIVATIONS``) the rows of w alternate gate and up rows and the
+    result is act(x.w[2j]) * (x.w[2j+1]) of width N/2 (an epilogue of the streaming kernels, a kernel
+    of its own after the library's product).
     """
     scale = None
     if isinstance(x, UnscaledRows):
@@ -548,7 +557,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
         y = gemm_f32(x, w)
     else:
         _need(x.dtype == w.dtype, "x and w must have one type")
-        plan = streaming_plan(x.shape[0], w.shape[0], w.shape[1], silu_pairs,
+        plan = streaming_plan(x.shape[0], w.shape[0], w.shape[1], bool(gate_pairs),
                               partial_ok and out_dtype in (None, torch.bfloat16), x.device, partial_max_width)
         _need(scale is None or (plan is not None and plan[0][0] == -2),
               "un-normalised rows need a product by the blocks that stay (ask linear_takes_unscaled_rows first)")
@@ -558,22 +567,22 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype=None, partial_ok: bool = 
                 return gemm_tile64(x, w, torch.float32, ksplit=parts)
             if parts > 1:
                 return gemm_skinny(x, w, torch.float32, block_shape=shape, ksplit=parts, row_scale=scale)
-            return gemm_skinny(x, w, out_dtype or torch.bfloat16, silu_pairs=silu_pairs, block_shape=shape,
+            return gemm_skinny(x, w, out_dtype or torch.bfloat16, gate_pairs=gate_pairs, block_shape=shape,
                                row_scale=scale)
         y = torch.mm(x, w.t())
-    if silu_pairs:
-        return silu_mul(y, interleaved=True)
+    if gate_pairs:
+        return gated_mul(y, interleaved=True, activation=gate_pairs)
     if out_dtype is not None and y.dtype != out_dtype:
         y = y.to(out_dtype)
     return y
 
 
-def linear_takes_unscaled_rows(n_rows: int, w: torch.Tensor, silu_pairs: bool = False, partial_ok: bool = False,
+def linear_takes_unscaled_rows(n_rows: int, w: torch.Tensor, gate_pairs: bool = False, partial_ok: bool = False,
                                partial_max_width: int | None = PARTIAL_SUM_MAX_WIDTH) -> bool:
     """Whether ``linear`` with these arguments multiplies ``UnscaledRows`` (its plan is the blocks that stay)."""
     if w.dtype != torch.bfloat16 or not unscaled_rows_possible(torch.bfloat16, n_rows, w.shape[1]):
         return False
-    plan = streaming_plan(n_rows, w.shape[0], w.shape[1], silu_pairs, partial_ok, w.device, partial_max_width)
+    plan = streaming_plan(n_rows, w.shape[0], w.shape[1], bool(gate_pairs), partial_ok, w.device, partial_max_width)
     return plan is not None and plan[0] != TILE64 and plan[0][0] == -2
 
 

@@ -1,5 +1,6 @@
-"""Gated feed-forward (SwiGLU).  Reference: ``jllm/model/common.py:69-76``:
-``down( silu(gate(x)) * up(x) )``, no biases.  gate and up are one matrix product against
+"""Gated feed-forward.  Reference: ``jllm/model/common.py:69-76``:
+``down( silu(gate(x)) * up(x) )``, no biases (SwiGLU); the gate's activation is a parameter, one
+of ``ops.kernels.GATE_ACTIVATIONS``.  gate and up are one matrix product against
 one weight whose rows alternate gate row j, up row j, so that a gate value and its up value
 come out next to each other: for few rows the activation is that product's epilogue, for
 many rows a kernel over adjacent pairs.  The activation runs in float."""
@@ -15,9 +16,10 @@ class GatedMLP:
     replayable = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
-        if activation != "silu":
-            raise ValueError(f"GatedMLP has kernels for 'silu' only, not {activation!r}")
+        if activation not in K.GATE_ACTIVATIONS:
+            raise ValueError(f"GatedMLP has kernels for {sorted(K.GATE_ACTIVATIONS)}, not for {activation!r}")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation = activation
         self.w_gate_up = self.w_down = None
 
     def tensors(self) -> dict:
@@ -35,10 +37,10 @@ class GatedMLP:
 
     def takes_unscaled_rows(self, n_rows: int) -> bool:
         """x goes into the gate/up product and nowhere else: the norm before may leave its scale to that product."""
-        return K.linear_takes_unscaled_rows(n_rows, self.w_gate_up, silu_pairs=True)
+        return K.linear_takes_unscaled_rows(n_rows, self.w_gate_up, gate_pairs=True)
 
     def forward(self, x, ctx=None) -> torch.Tensor:
-        z = K.linear(x, self.w_gate_up, silu_pairs=True)    # gate and up rows alternate in the fused weight
+        z = K.linear(x, self.w_gate_up, gate_pairs=self.activation)    # gate and up rows alternate in the fused weight
         return K.linear(z, self.w_down, partial_ok=True)   # the next norm adds the partial products
 
 

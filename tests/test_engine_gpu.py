@@ -486,6 +486,20 @@ def test_parts_alone(dtype):
             assert got.dtype == torch.float32
             got = got.sum(0)
         torch.testing.assert_close(got.float().cpu(), ref, **tol)
+    # the gate's activation is a parameter of the part: the tanh form of gelu against the library's
+    gelu = build_part("feed_forward", PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter,
+                                                            "activation": "gelu_tanh"}))
+    gelu.bind({k: v.cuda() for k, v in ws.items()}, dtype)
+    for rows in (t, 40, 70):   # epilogue of the streaming kernels, of the 64-row tiles, kernel after the library
+        xi = torch.randn(rows, hidden, generator=g).to(dtype)
+        gate = torch.nn.functional.gelu(xi.float() @ ws["gate_proj.weight"].float().T, approximate="tanh")
+        ref = (gate * (xi.float() @ ws["up_proj.weight"].float().T)) @ ws["down_proj.weight"].float().T
+        got = gelu.forward(xi.cuda())
+        got = got.sum(0) if got.dim() == 3 else got
+        torch.testing.assert_close(got.float().cpu(), ref, **tol)
+    with pytest.raises(ValueError, match="gelu_tanh"):
+        build_part("feed_forward", PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter,
+                                                          "activation": "relu"}))
 
     emb = build_part("embedding", PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": hidden}))
     table = torch.randn(vocab, hidden, generator=g).to(dtype)

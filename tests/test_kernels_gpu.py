@@ -75,17 +75,28 @@ def test_rmsnorm_last_axis(dtype):
     torch.testing.assert_close(out.float(), ref, **tol(dtype))
 
 
+def gate_activation(name, g):
+    """The library routine a gate activation of the kernels reduces to."""
+    return torch.nn.functional.silu(g) if name == "silu" else torch.nn.functional.gelu(g, approximate="tanh")
+
+
+ACTIVATIONS = ["silu", "gelu_tanh"]
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("inter", [176, 12288, 77])
-def test_silu_mul(dtype, inter):
+@pytest.mark.parametrize("act", ACTIVATIONS)
+def test_gated_mul(dtype, inter, act):
     gu = randn(9, 2 * inter, dtype=dtype, seed=6, scale=3.0)
-    out = K().silu_mul(gu)
+    out = K().gated_mul(gu, activation=act)
     g, u = gu.float()[:, :inter], gu.float()[:, inter:]
-    torch.testing.assert_close(out.float(), torch.nn.functional.silu(g) * u, **tol(dtype))
+    torch.testing.assert_close(out.float(), gate_activation(act, g) * u, **tol(dtype))
     # gate and up alternating along the row
-    out2 = K().silu_mul(gu, interleaved=True)
+    out2 = K().gated_mul(gu, interleaved=True, activation=act)
     g2, u2 = gu.float()[:, 0::2], gu.float()[:, 1::2]
-    torch.testing.assert_close(out2.float(), torch.nn.functional.silu(g2) * u2, **tol(dtype))
+    torch.testing.assert_close(out2.float(), gate_activation(act, g2) * u2, **tol(dtype))
+    with pytest.raises(ValueError):
+        K().gated_mul(gu, activation="relu")
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 50, 70), (5, 333, 80), (70, 130, 257), (130, 64, 16)])
@@ -803,14 +814,17 @@ def test_gemm_tile64(m, n, k, ksplit):
     torch.testing.assert_close(K().gemm_tile64(x, w, out_dtype, ksplit=ksplit), y, rtol=0, atol=0)
 
 
-def test_gemm_tile64_silu_epilogue_and_refusals():
+@pytest.mark.parametrize("act", ACTIVATIONS)
+def test_gemm_tile64_activation_epilogue_and_refusals(act):
     x = randn(40, 1024, dtype=torch.bfloat16, seed=53, scale=0.5)
     w = randn(300, 1024, dtype=torch.bfloat16, seed=54, scale=0.1)
     g, u = w[0::2].double(), w[1::2].double()
-    want = torch.nn.functional.silu(x.double() @ g.T) * (x.double() @ u.T)
-    got = K().gemm_tile64(x, w, silu_pairs=True)
+    want = gate_activation(act, x.double() @ g.T) * (x.double() @ u.T)
+    got = K().gemm_tile64(x, w, gate_pairs=act)
     assert got.shape == (40, 150)
     torch.testing.assert_close(got.double(), want, rtol=2e-2, atol=2e-2)
+    with pytest.raises(ValueError):
+        K().gemm_tile64(x, w, gate_pairs="relu")                                    # no such kernel
     with pytest.raises(ValueError):
         K().gemm_tile64(randn(65, 1024, dtype=torch.bfloat16), w)                    # more than 64 rows
     with pytest.raises(ValueError):
@@ -818,7 +832,7 @@ def test_gemm_tile64_silu_epilogue_and_refusals():
     with pytest.raises(ValueError):
         K().gemm_tile64(x, w, torch.bfloat16, ksplit=2)                             # partial products are float32
     with pytest.raises(ValueError):
-        K().gemm_tile64(x, w, silu_pairs=True, ksplit=2, out_dtype=torch.float32)   # no activation of a partial sum
+        K().gemm_tile64(x, w, gate_pairs=act, ksplit=2, out_dtype=torch.float32)   # no activation of a partial sum
 
 
 @pytest.mark.parametrize("m,hidden,n_parts", [(8, 4096, 4), (1, 512, 2), (16, 5120, 3), (5, 8192, 1)])
@@ -852,8 +866,8 @@ def test_residual_step_that_leaves_the_scale_to_the_product(m, hidden, n_parts):
         y = y.sum(0) if y.dim() == 3 else y.float()
         torch.testing.assert_close(y.double(), xn @ w.double().T, rtol=2e-2, atol=2e-2)
     wide = randn(2 * 16 * 4 * 256, hidden, dtype=torch.bfloat16, seed=74, scale=0.05)     # 1,024 row tiles: the wide plan
-    if kern.linear_takes_unscaled_rows(m, wide, silu_pairs=True):
-        z = kern.linear(rows, wide, silu_pairs=True)
+    if kern.linear_takes_unscaled_rows(m, wide, gate_pairs=True):
+        z = kern.linear(rows, wide, gate_pairs="silu")
         full = xn @ wide.double().T
         gate, up = full[:, 0::2], full[:, 1::2]
         torch.testing.assert_close(z.double(), gate / (1 + torch.exp(-gate)) * up, rtol=3e-2, atol=3e-2)
@@ -912,7 +926,7 @@ def test_linear_at_every_size_runs_a_plan_the_library_accepts(k):
             y = y.sum(0) if y.dim() == 3 else y
             torch.testing.assert_close(y.double(), ref, **tol_)
             torch.testing.assert_close(kern.linear(x, w).double(), ref, **tol_)
-            act = kern.linear(x, w, silu_pairs=True)
+            act = kern.linear(x, w, gate_pairs="silu")
             want = torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2]
             torch.testing.assert_close(act.double(), want, rtol=3e-2, atol=3e-2 * math.sqrt(k) / 8)
 
@@ -924,7 +938,7 @@ def test_linear_follows_its_plan_and_all_roads_agree():
     x = randn(8, 4096, dtype=torch.bfloat16, seed=36, scale=0.5)
     wide = randn(16640, 4096, dtype=torch.bfloat16, seed=37, scale=0.1)      # 1,040 row tiles: blocks that stay
     narrow = randn(512, 4096, dtype=torch.bfloat16, seed=38, scale=0.1)      # 32 row tiles: inner size shared out
-    assert kern.streaming_plan(8, 16640, 4096, silu_pairs=True, device=x.device)[0][0] == -2
+    assert kern.streaming_plan(8, 16640, 4096, gate_pairs=True, device=x.device)[0][0] == -2
     plan = kern.streaming_plan(8, 512, 4096, partial_ok=True, device=x.device)
     assert plan[1] == 4 and kern.streaming_plan(8, 512, 4096, partial_ok=False, device=x.device) == ((0, 0, 0), 1)
     assert kern.streaming_plan(17, 512, 4096, device=x.device) is None       # the library's
@@ -938,7 +952,7 @@ def test_linear_follows_its_plan_and_all_roads_agree():
     for rows in (8, 40):                                                    # staying blocks; library + silu kernel
         xi = x if rows == 8 else randn(rows, 4096, dtype=torch.bfloat16, seed=39, scale=0.5)
         want = ref_act if rows == 8 else torch.nn.functional.silu(xi.double() @ g.T) * (xi.double() @ u.T)
-        got = kern.linear(xi, wide, silu_pairs=True)
+        got = kern.linear(xi, wide, gate_pairs="silu")
         assert got.shape == (rows, 8320) and got.dtype == torch.bfloat16
         torch.testing.assert_close(got.double(), want, rtol=2e-2, atol=5e-2)
 
@@ -946,13 +960,14 @@ def test_linear_follows_its_plan_and_all_roads_agree():
 @pytest.mark.parametrize("m,inter,k,shape", [(1, 176, 80, (0, 0, 0)), (8, 12288, 96, (0, 0, 0)), (40, 224, 104, (0, 0, 0)),
                                              (16, 1000, 4096, (0, 0, 0)), (8, 1000, 4096, (-2, 256, 16)),
                                              (3, 177, 1000, (-2, 5, 4))])
-def test_gemm_skinny_silu_epilogue(m, inter, k, shape):
-    """Rows of w alternate gate and up rows; the product comes out as silu(gate) * up."""
+@pytest.mark.parametrize("act", ACTIVATIONS)
+def test_gemm_skinny_activation_epilogue(m, inter, k, shape, act):
+    """Rows of w alternate gate and up rows; the product comes out as act(gate) * up."""
     x = randn(m, k, dtype=torch.bfloat16, seed=32, scale=0.7)
     wg = randn(inter, k, dtype=torch.bfloat16, seed=33, scale=0.3)
     wu = randn(inter, k, dtype=torch.bfloat16, seed=34, scale=0.3)
     w = torch.stack([wg, wu], dim=1).reshape(2 * inter, k).contiguous()
-    out = K().gemm_skinny(x, w, torch.bfloat16, silu_pairs=True, block_shape=shape)
+    out = K().gemm_skinny(x, w, torch.bfloat16, gate_pairs=act, block_shape=shape)
     assert out.shape == (m, inter)
-    ref = torch.nn.functional.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
+    ref = gate_activation(act, x.double() @ wg.double().T) * (x.double() @ wu.double().T)
     torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=2e-2 * math.sqrt(k) / 4)

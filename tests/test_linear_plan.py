@@ -41,7 +41,7 @@ def acceptable(m, n, k, silu, plan):
 @pytest.mark.parametrize("silu,partial_ok", [(False, False), (False, True), (True, False)])
 def test_every_plan_is_one_the_kernels_accept(silu, partial_ok):
     for m, n, k in itertools.product(ROWS, WIDTHS, INNER):
-        plan = K.streaming_plan(m, n, k, silu_pairs=silu, partial_ok=partial_ok)
+        plan = K.streaming_plan(m, n, k, gate_pairs=silu, partial_ok=partial_ok)
         if plan is None:
             continue                        # the library's
         assert m <= 64 and k % 8 == 0
@@ -56,7 +56,7 @@ def test_plans_at_the_sizes_they_were_measured_at():
     plan = K.streaming_plan
     assert plan(8, 4096, 4096, partial_ok=True) == ((-2, 512, 4), 4)            # o_proj, 8B
     assert plan(8, 4096, 12288, partial_ok=True) == ((-2, 256, 12), 4)          # down_proj, 8B
-    assert plan(8, 24576, 4096, silu_pairs=True) == ((-2, 256, 16), 1)          # gate and up, 8B
+    assert plan(8, 24576, 4096, gate_pairs=True) == ((-2, 256, 16), 1)          # gate and up, 8B
     assert plan(64, 4096, 12288, partial_ok=True) == (K.TILE64, 4)              # down_proj at 64 rows
     assert plan(64, 5120, 17408, partial_ok=True) == (K.TILE64, 3)              # 80 tiles of 64 rows: 3 groups fill 256 units
     assert plan(64, 4096, 4096, partial_ok=True) == ((-2, 256, 4), 4)           # four row tiles of x in registers
@@ -66,8 +66,8 @@ def test_plans_at_the_sizes_they_were_measured_at():
     assert plan(8, 1024, 3072, partial_ok=True) == ((-2, 512, 8), 2)            # no piece count covers 3,072 with 4 groups
     assert plan(8, 5120, 25600, partial_ok=True) == (K.PARTIAL_SHAPE, 4)        # none with 2 or 4: x resident in LDS
     assert plan(8, 1024, 1000 * 8, partial_ok=True)[1] in (2, 3, 4)
-    assert plan(8, 34816, 5120, silu_pairs=True) == ((-2, 256, 20), 1)          # gate and up, 14B
-    assert plan(1, 24576, 4096, silu_pairs=True) == ((-2, 256, 16), 1)          # one row: the same blocks
+    assert plan(8, 34816, 5120, gate_pairs=True) == ((-2, 256, 20), 1)          # gate and up, 14B
+    assert plan(1, 24576, 4096, gate_pairs=True) == ((-2, 256, 16), 1)          # one row: the same blocks
     assert plan(8, 10240, 5120, partial_ok=True) == ((0, 0, 0), 1)              # wider than the norm adds parts of ...
     assert plan(8, 10240, 5120, partial_ok=True, partial_max_width=None) == ((-2, 256, 5), 4)   # ... but the rotation kernel does
     assert plan(8, 4096, 4100) is None                                          # inner size no multiple of 8
