@@ -343,6 +343,16 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
   for (int c = threadIdx.x; c < n; c += blockDim.x) out[i * n + c] = from_f32<T>(x[r * n + c]);
 }
 
+// ---------------------------------------------------------------- bias of a projection
+// y[r, c] += bias[c], summed in float; grid (column blocks, rows)
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bias, int n) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n) return;
+  T* at = y + (long long)blockIdx.y * n + c;
+  *at = from_f32<T>(to_f32(*at) + bias[c]);
+}
+
 #define DEFINE_ELEMENTWISE(SUF, T)                                                                  \
   extern "C" int jv_embedding_##SUF(float* h, const void* table, const int* ids, int n_tokens,      \
                                     int hidden, void* stream) {                                     \
@@ -434,6 +444,15 @@ __global__ void cast_rows_kernel(T* __restrict__ out, const float* __restrict__ 
     if (n_out <= 0) return 0;                                                                       \
     hipLaunchKernelGGL(cast_rows_kernel<T>, dim3(n_out), dim3(256), 0, (hipStream_t)stream,         \
                        (T*)out, x, rows, n);                                                        \
+    return JV_LAUNCH_CHECK();                                                                       \
+  }                                                                                                 \
+  extern "C" int jv_add_bias_##SUF(void* y, const float* bias, long long rows, int n, void* stream) { \
+    if (rows <= 0 || n <= 0) return 0;                                                              \
+    for (long long r0 = 0; r0 < rows; r0 += 65535) { /* grid.y limit */                             \
+      const unsigned ny = (unsigned)(rows - r0 < 65535 ? rows - r0 : 65535);                        \
+      hipLaunchKernelGGL(add_bias_kernel<T>, dim3((n + 255) / 256, ny), dim3(256), 0,               \
+                         (hipStream_t)stream, (T*)y + r0 * n, bias, n);                             \
+    }                                                                                               \
     return JV_LAUNCH_CHECK();                                                                       \
   }
 

@@ -188,6 +188,17 @@ def cast_rows(x: torch.Tensor, dtype: torch.dtype, rows=None) -> torch.Tensor:
     return out
 
 
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
+    """y[..., c] += bias[c] in place, for what ``linear`` returned: rows [M, N], or a float stack [parts, M, N]
+    of partial products, of which the first takes the bias."""
+    _dev(y, bias)
+    rows = y[0] if y.dim() == 3 else y
+    _need(rows.dim() == 2 and rows.is_contiguous() and bias.is_contiguous(), "y must be contiguous rows")
+    _f32(bias, "bias", rows.shape[1])
+    fn = getattr(library.core(), f"jv_add_bias_{_suffix(rows.dtype)}")
+    _check(fn(_ptr(rows), _ptr(bias), c_longlong(rows.shape[0]), c_int(rows.shape[1]), _stream()), "add_bias")
+
+
 # --------------------------------------------------------------------------- activation
 GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}      # the kernels' ids of act in y = act(gate) * up
 

@@ -53,18 +53,26 @@ def _hipcc() -> str:
     raise KernelLibraryError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
 
 
+_build_dir: "Path | None" = None
+_build_dir_lock = threading.Lock()
+
+
 def build_dir() -> Path:
-    d = CSRC / "_build"
-    try:
-        d.mkdir(exist_ok=True)
-        probe = d / f".w{os.getpid()}"
-        probe.write_text("")
-        probe.unlink()
-        return d
-    except OSError:
-        d = Path(tempfile.gettempdir()) / f"jax_vllm_amd_build_{os.getuid()}"
-        d.mkdir(parents=True, exist_ok=True)
-        return d
+    """Where the libraries live: decided once per process (the parallel builds all ask)."""
+    global _build_dir
+    with _build_dir_lock:
+        if _build_dir is None:
+            d = CSRC / "_build"
+            try:
+                d.mkdir(exist_ok=True)
+                probe = d / f".w{os.getpid()}"
+                probe.write_text("")
+                probe.unlink(missing_ok=True)
+            except OSError:
+                d = Path(tempfile.gettempdir()) / f"jax_vllm_amd_build_{os.getuid()}"
+                d.mkdir(parents=True, exist_ok=True)
+            _build_dir = d
+        return _build_dir
 
 
 def _core_sources() -> list[Path]:

@@ -1,7 +1,8 @@
 """Grouped-query causal attention over a paged cache: the token mixer of Qwen3.
 
 Reference: ``jllm/model/common.py:114-137`` (projections, head layout, output
-projection), ``:107-111`` (optional per-head q/k RMSNorm before the rotation),
+projection; the reference's projections have no bias, here ``qkv_bias`` and ``o_bias`` are options of the
+part), ``:107-111`` (optional per-head q/k RMSNorm before the rotation),
 ``:173-214`` (scores, mask, softmax, kv head = q head // group).  The three input
 projections are one matrix product against the row-concatenated weight; scores,
 mask and softmax are float inside the attention kernels; keys are stored after
@@ -22,7 +23,8 @@ from .spec import (KVCacheSpec, LayerMemory, PartSpec, StepContext, TensorSpec, 
 class GroupedQueryAttention:
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  qk_norm_eps: Optional[float] = None, position: Optional[PartSpec] = None,
-                 window: Optional[int] = None, scale: Optional[float] = None):
+                 window: Optional[int] = None, scale: Optional[float] = None, qkv_bias: bool = False,
+                 o_bias: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} q heads are not a multiple of {num_kv_heads} kv heads")
         self.hidden_size, self.nq, self.nkv, self.d = int(hidden_size), int(num_heads), int(num_kv_heads), int(head_dim)
@@ -30,7 +32,8 @@ class GroupedQueryAttention:
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
         self.position = build_part("position", position) if position is not None else None
-        self.w_qkv = self.w_o = self.q_norm = self.k_norm = None
+        self.qkv_bias, self.o_bias = bool(qkv_bias), bool(o_bias)
+        self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.b_qkv = self.b_o = None
 
     # ---- declarations
     @property
@@ -50,6 +53,12 @@ class GroupedQueryAttention:
         if self.qk_norm_eps is not None:
             t["q_norm.weight"] = TensorSpec((self.d,), role="vector", init="norm")
             t["k_norm.weight"] = TensorSpec((self.d,), role="vector", init="norm")
+        if self.qkv_bias:
+            t["q_proj.bias"] = TensorSpec((self.nq * self.d,), role="vector")
+            t["k_proj.bias"] = TensorSpec((self.nkv * self.d,), role="vector")
+            t["v_proj.bias"] = TensorSpec((self.nkv * self.d,), role="vector")
+        if self.o_bias:
+            t["o_proj.bias"] = TensorSpec((self.hidden_size,), role="vector")
         return t
 
     def cache_spec(self) -> Optional[KVCacheSpec]:
@@ -66,6 +75,10 @@ class GroupedQueryAttention:
         self.w_o = tensors["o_proj.weight"]
         if self.qk_norm_eps is not None:
             self.q_norm, self.k_norm = tensors["q_norm.weight"], tensors["k_norm.weight"]
+        if self.qkv_bias:
+            self.b_qkv = torch.cat([tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]]).contiguous()
+        if self.o_bias:
+            self.b_o = tensors["o_proj.bias"].contiguous()
         if self.position is not None:
             self.position.bind({}, dtype, self.w_o.device)
 
@@ -88,6 +101,8 @@ class GroupedQueryAttention:
         # at few rows the projection may come as float partial products, which the next kernel adds
         qkv = K.linear(x, self.w_qkv, partial_max_width=None,       # the rotation kernel adds parts of any width
                        partial_ok=K.rope_takes_parts(x.dtype, self.d, interleaved, rotary_dim, cos_sin is not None))
+        if self.b_qkv is not None:
+            K.add_bias(qkv, self.b_qkv)
         parts = None
         if qkv.dim() == 3:
             parts, qkv = qkv, torch.empty(qkv.shape[1:], dtype=x.dtype, device=x.device)
@@ -102,7 +117,10 @@ class GroupedQueryAttention:
         from . import attention_backend
 
         attention_backend.run(self, out, qkv, ctx, mem)
-        return K.linear(out, self.w_o, partial_ok=True)   # the next norm adds the partial products
+        y = K.linear(out, self.w_o, partial_ok=True)      # the next norm adds the partial products
+        if self.b_o is not None:
+            K.add_bias(y, self.b_o)
+        return y
 
 
 register_part("mixer", "gqa_attention", GroupedQueryAttention)

@@ -524,9 +524,12 @@ def test_parts_alone(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_attention_part_alone(folders, dtype):
+@pytest.mark.parametrize("biased", [False, True])
+def test_attention_part_alone(folders, dtype, biased):
     """The mixer with its cache, outside any model: two portions of one request and a second
-    request beside it, against the plain attention block."""
+    request beside it, against the plain attention block.  ``biased``: the part's options
+    ``qkv_bias`` and ``o_bias``; a bias is one more input column that is always 1, so the plain
+    block gives the reference with the bias as a last column of its weight."""
     from jax_vllm_amd.cache import CacheManager
     from jax_vllm_amd.cache.storage import allocate_memories
     from jax_vllm_amd.parts import KVCacheSpec, PartSpec, build_part
@@ -538,8 +541,10 @@ def test_attention_part_alone(folders, dtype):
     g = torch.Generator().manual_seed(12)
     att = build_part("mixer", PartSpec("gqa_attention", dict(
         hidden_size=hidden, num_heads=nq, num_kv_heads=nkv, head_dim=d, qk_norm_eps=1e-5,
-        position=PartSpec("rotary", {"head_dim": d, "theta": 1e4}))))
-    ws = {n: ((0.15 * torch.randn(s.shape, generator=g)) if s.role == "matrix" else 1 + 0.1 * torch.randn(s.shape, generator=g))
+        position=PartSpec("rotary", {"head_dim": d, "theta": 1e4}), qkv_bias=biased, o_bias=biased)))
+    assert ("q_proj.bias" in att.tensors()) == biased and ("o_proj.bias" in att.tensors()) == biased
+    ws = {n: ((0.15 * torch.randn(s.shape, generator=g)) if s.role == "matrix" else
+              0.3 * torch.randn(s.shape, generator=g) if n.endswith(".bias") else 1 + 0.1 * torch.randn(s.shape, generator=g))
           for n, s in att.tensors().items()}
     ws = {n: v.to(tdt).float() for n, v in ws.items()}
     att.bind({n: v.to(tdt if att.tensors()[n].role == "matrix" else torch.float32).cuda() for n, v in ws.items()}, tdt)
@@ -550,8 +555,15 @@ def test_attention_part_alone(folders, dtype):
     cfg = dict(num_heads=nq, num_kv_heads=nkv, head_dim=d, rms_norm_eps=1e-5, rope_theta=1e4)
     xa, xb = torch.randn(21, hidden, generator=g).to(tdt), torch.randn(5, hidden, generator=g).to(tdt)
     pw = {f"p.{n}": v for n, v in ws.items()}
-    want_a = P.attention_block(pw, "p", cfg, xa.float(), torch.arange(21))
-    want_b = P.attention_block(pw, "p", cfg, xb.float(), torch.arange(5))
+    one = lambda x: x.float()
+    if biased:
+        for n in ("q_proj", "k_proj", "v_proj"):
+            pw[f"p.{n}.weight"] = torch.cat([ws[f"{n}.weight"], ws[f"{n}.bias"][:, None]], dim=1)
+        one = lambda x: torch.cat([x.float(), torch.ones(x.shape[0], 1)], dim=1)
+    want_a = P.attention_block(pw, "p", cfg, one(xa), torch.arange(21))
+    want_b = P.attention_block(pw, "p", cfg, one(xb), torch.arange(5))
+    if biased:
+        want_a, want_b = want_a + ws["o_proj.bias"], want_b + ws["o_proj.bias"]
     cache.start("a"), cache.start("b")
 
     def step(parts):
