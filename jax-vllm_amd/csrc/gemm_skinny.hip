@@ -350,7 +350,13 @@ struct RowScale {
 // its end): rows of W beyond N read the last row (their outputs are never stored), rows of x beyond M read
 // the last row (likewise); EDGE (the inner size is not ksplit * 8 * NL * 32 exactly): columns beyond K read
 // the row's last piece again, against zeros in x.
-template <int NL, int MT, typename OutT, bool PAIRS, bool EDGE>
+//
+// SLOTS > 0 (a divisor of NL): instead of two whole tiles that take turns, W sits in SLOTS slots of NL / SLOTS
+// pieces; part q of every tile goes through slot q, which is filled with the next tile's part as soon as it has
+// been multiplied, so all slots but one are in flight.  With 4 slots that is three quarters of a tile on its way
+// in half the registers of the two-tile scheme: what two row tiles of x with 16 pieces a wave need to fit (128
+// registers of x, 64 of W).
+template <int NL, int MT, typename OutT, bool PAIRS, bool EDGE, int SLOTS = 0>
 __global__ void __launch_bounds__(512)
 gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
                               int M, int N, int K, long long ldx, long long ldy, RowScale rs) {
@@ -385,23 +391,29 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
     const float* sp = rs.ssq ? rs.ssq + (long long)m * 16 + lc * 4 : (const float*)x;
     row_sq = *(const f32x4*)sp;
   }
-  auto load_tile = [&](int tile, bf16x8 (&a)[NL]) {
+  // pieces first .. first + CNT - 1 of a tile
+  auto load_pieces = [&](int tile, int first, auto& a) {
+    constexpr int CNT = sizeof(a) / sizeof(a[0]);
     const int n = min(tile * 16 + li, N - 1);
     const bool real = tile < n_tiles;
     const bf16_t* wrow = W + (real ? (long long)n * K : 0);
-    const int kk = real ? k0 : 0;
+    const int kk = (real ? k0 : 0) + first * 32;
 #pragma unroll
-    for (int i = 0; i < NL; ++i) a[i] = *(const bf16x8*)(wrow + (EDGE ? min(kk + i * 32, K - 8) : kk + i * 32));
+    for (int i = 0; i < CNT; ++i) a[i] = *(const bf16x8*)(wrow + (EDGE ? min(kk + i * 32, K - 8) : kk + i * 32));
   };
-  auto finish_tile = [&](int tile, bf16x8 (&a)[NL], int buf) {
-    f32x4 acc[MT];
+  auto load_tile = [&](int tile, bf16x8 (&a)[NL]) { load_pieces(tile, 0, a); };
+  auto multiply_pieces = [&](int first, const auto& a, f32x4 (&acc)[MT]) {
+    constexpr int CNT = sizeof(a) / sizeof(a[0]);
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-      for (int i = 0; i < NL; ++i) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[mt][i], acc[mt], 0, 0, 0);
-      *(f32x4*)(red[buf] + ((wk * MT + mt) * 256 + lane * 4)) = acc[mt];
-    }
+      for (int i = 0; i < CNT; ++i)
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[mt][first + i], acc[mt], 0, 0, 0);
+  };
+  // the 8 waves' sums of a tile, added in fixed order and stored
+  auto reduce_store = [&](int tile, const f32x4 (&acc)[MT], int buf) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) *(f32x4*)(red[buf] + ((wk * MT + mt) * 256 + lane * 4)) = acc[mt];
     __syncthreads();
     if (wk < MT) {                                 // wave mt adds row tile mt, in fixed order: wave 0, 1, ..., 7
       const int mt = wk;
@@ -439,49 +451,82 @@ gemm_skinny_persistent_kernel(OutT* __restrict__ y, const bf16_t* __restrict__ x
   // The next tile's weights are asked for before this tile is multiplied, without a condition (beyond the
   // last tile the last one is read again): after a conditional prefetch the compiler must assume that
   // nothing younger is in flight, and its wait for this tile's first piece then waits for the prefetch too.
-  bf16x8 a0[NL], a1[NL];
   int tile = blockIdx.x;                             // the launch has no more blocks than tiles
-  load_tile(tile, a0);
-  for (;;) {
-    int next = tile + gridDim.x;
-    __builtin_amdgcn_sched_barrier(0);
-    load_tile(next, a1);
-    __builtin_amdgcn_sched_barrier(0);
-    finish_tile(tile, a0, 0);
-    if (next >= n_tiles) break;
-    tile = next;
-    next = tile + gridDim.x;
-    __builtin_amdgcn_sched_barrier(0);
-    load_tile(next, a0);
-    __builtin_amdgcn_sched_barrier(0);
-    finish_tile(tile, a1, 1);
-    if (next >= n_tiles) break;
-    tile = next;
+  if constexpr (SLOTS == 0) {
+    auto finish_tile = [&](int t, bf16x8 (&a)[NL], int buf) {
+      f32x4 acc[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      multiply_pieces(0, a, acc);
+      reduce_store(t, acc, buf);
+    };
+    bf16x8 a0[NL], a1[NL];
+    load_tile(tile, a0);
+    for (;;) {
+      int next = tile + gridDim.x;
+      __builtin_amdgcn_sched_barrier(0);
+      load_tile(next, a1);
+      __builtin_amdgcn_sched_barrier(0);
+      finish_tile(tile, a0, 0);
+      if (next >= n_tiles) break;
+      tile = next;
+      next = tile + gridDim.x;
+      __builtin_amdgcn_sched_barrier(0);
+      load_tile(next, a0);
+      __builtin_amdgcn_sched_barrier(0);
+      finish_tile(tile, a1, 1);
+      if (next >= n_tiles) break;
+      tile = next;
+    }
+  } else {
+    static_assert(SLOTS == 0 || NL % (SLOTS ? SLOTS : 1) == 0, "a slot holds a whole number of pieces");
+    constexpr int S = NL / (SLOTS ? SLOTS : 1);
+    bf16x8 slot[SLOTS ? SLOTS : 1][S];
+#pragma unroll
+    for (int q = 0; q < SLOTS; ++q) load_pieces(tile, q * S, slot[q]);
+    for (int buf = 0;; buf ^= 1) {
+      const int next = tile + gridDim.x;
+      f32x4 acc[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int q = 0; q < SLOTS; ++q) {
+        __builtin_amdgcn_sched_barrier(0);
+        multiply_pieces(q * S, slot[q], acc);
+        __builtin_amdgcn_sched_barrier(0);
+        load_pieces(next, q * S, slot[q]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      reduce_store(tile, acc, buf);
+      if (next >= n_tiles) break;
+      tile = next;
+    }
   }
 }
 
-template <int NL, int MT, typename OutT, bool PAIRS>
+template <int NL, int MT, typename OutT, bool PAIRS, int SLOTS = 0>
 static int launch_persistent(void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
                              long long ldy, int blocks, int ksplit, RowScale rs, hipStream_t stream) {
   const int n_tiles = (N + 15) / 16;
   blocks = (blocks + ksplit - 1) / ksplit;           // per group
   if (blocks > n_tiles) blocks = n_tiles;
   if (K == ksplit * 8 * NL * 32)
-    hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, false>), dim3(blocks, ksplit), dim3(512), 0,
+    hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, false, SLOTS>), dim3(blocks, ksplit), dim3(512), 0,
                        stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, rs);
   else
-    hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, true>), dim3(blocks, ksplit), dim3(512), 0,
+    hipLaunchKernelGGL((gemm_skinny_persistent_kernel<NL, MT, OutT, PAIRS, true, SLOTS>), dim3(blocks, ksplit), dim3(512), 0,
                        stream, (OutT*)y, (const bf16_t*)x, (const bf16_t*)W, M, N, K, ldx, ldy, rs);
   return JV_LAUNCH_CHECK();
 }
 
 // wr == -2: nks = NL in {4, 5, 8, 10, 12, 16, 17, 20}, wk = blocks in all; the inner size must be at most
 // ksplit * 8 * NL * 32 and more than (ksplit - 1) * 8 * NL * 32.  Up to 16 rows with every NL, up
-// to 32 rows (two row tiles of x in registers) with NL <= 8.
+// to 32 rows (two row tiles of x in registers) with NL <= 8 and, W in slots, with NL 12 and 16;
+// up to 64 rows with NL <= 5.
 template <typename OutT, bool PAIRS>
 static int dispatch_persistent(int nl, void* y, const void* x, const void* W, int M, int N, int K, long long ldx,
                                long long ldy, int blocks, int ksplit, RowScale rs, hipStream_t s) {
-  if (M > 64 || (M > 16 && nl > 8) || (M > 32 && nl > 5) || blocks < 1 || ksplit > 65535 ||
+  if (M > 64 || (M > 16 && nl > 16) || (M > 32 && nl > 5) || blocks < 1 || ksplit > 65535 ||
       K > (long long)ksplit * 8 * nl * 32 || K <= (long long)(ksplit - 1) * 8 * nl * 32)
     return (int)hipErrorInvalidValue;
   if (M > 48) {
@@ -503,6 +548,8 @@ static int dispatch_persistent(int nl, void* y, const void* x, const void* W, in
       case 4: return launch_persistent<4, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
       case 5: return launch_persistent<5, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
       case 8: return launch_persistent<8, 2, OutT, PAIRS>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+      case 12: return launch_persistent<12, 2, OutT, PAIRS, 4>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
+      case 16: return launch_persistent<16, 2, OutT, PAIRS, 4>(y, x, W, M, N, K, ldx, ldy, blocks, ksplit, rs, s);
     }
     return (int)hipErrorInvalidValue;
   }

@@ -376,10 +376,11 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype=torch.bfloat16, gate
     _need(m <= SKINNY_MAX_ROWS, f"gemm_skinny takes at most {SKINNY_MAX_ROWS} rows")
     _need(k % 8 == 0, "the inner size must be a multiple of 8")
     _need(out_dtype in (torch.bfloat16, torch.float32), "output must be bfloat16 or float32")
-    _need(block_shape[0] != -2 or ((m <= 16 or (m <= 32 and block_shape[2] <= 8) or block_shape[2] <= 5) and block_shape[2] in STAY_PIECES
+    _need(block_shape[0] != -2 or ((m <= 16 or (m <= 32 and block_shape[2] in STAY_PIECES_32_ROWS) or block_shape[2] <= 5)
+                                   and block_shape[2] in STAY_PIECES
                                    and 256 * block_shape[2] * (ksplit - 1) < k <= 256 * block_shape[2] * ksplit),
-          "the organisation with blocks that stay takes at most 16 rows (32 with at most 8 pieces) and an inner "
-          "size of ksplit * 256 * pieces at most")
+          "the organisation with blocks that stay takes at most 16 rows (32 with at most 16 pieces, 64 with at most 5) "
+          "and an inner size of ksplit * 256 * pieces at most")
     _need(not gate_pairs or (out_dtype == torch.bfloat16 and n % 2 == 0 and block_shape[0] != -1),
           "the activation epilogue writes bfloat16, needs an even number of rows of w and the chunked organisation")
     _need(ksplit >= 1 and (ksplit == 1 or (block_shape[0] in (-1, -2) and out_dtype == torch.float32
@@ -454,7 +455,8 @@ def compute_units(device) -> int:
     return n
 
 
-STAY_PIECES = (4, 5, 8, 10, 12, 16, 17, 20)   # weight pieces per wave the staying blocks are built for
+STAY_PIECES = (4, 5, 8, 10, 12, 16, 17, 20)
+STAY_PIECES_32_ROWS = (4, 5, 8, 12, 16)      # of these, the ones built for 17..32 rows (two row tiles of x in registers)
 
 
 def _fit_parts(units: int, parts: int) -> int:
@@ -502,6 +504,10 @@ def streaming_plan(m: int, n: int, k: int, gate_pairs: bool = False, partial_ok:
       wave for two, 5 for more), the inner size shared out to 4 groups (4,096 x 4,096: 10.3 us at
       32 rows, 13.2 at 64, against the library's 13.0 and 15.0; 5,120 x 5,120 at 48 rows: 16.5
       against 26.6);
+    * 17..32 rows against wide matrices with an inner size of 12 or 16 pieces a wave (gate and up, the output
+      embedding): staying blocks with two row tiles of x in registers and W in four slots (24,576 x 4,096
+      with the activation at 24 rows 41.9 us, at 32 rows 43.7, against 47.5 and 47.2 by the library and the
+      activation kernel; 151,936 x 4,096 at 24 rows 248 against 270);
     * one or two rows against very wide matrices (the output embedding): x resident in LDS (chosen
       inside the kernel library; 1.24 GB in 202 us against 205);
     * 9..16 rows of a large matrix that fits none of these: the library (its wider tiles amortise
@@ -514,6 +520,10 @@ def streaming_plan(m: int, n: int, k: int, gate_pairs: bool = False, partial_ok:
     cus = compute_units(device) if device is not None else 256
     narrow = partial_ok and not gate_pairs and n % 4 == 0 and (partial_max_width is None or n <= partial_max_width)
     if m > SKINNY_AUTO_ROWS:
+        if m <= 32 and -(-n // 16) >= 4 * cus:
+            nl = _stay_pieces(k, 1)
+            if nl in (12, 16):
+                return (-2, cus, nl), 1
         if narrow and m <= SKINNY_MAX_ROWS:
             parts = _fit_parts(-(-k // 256), min(4, cus // -(-n // 64)))
             if parts >= 2 and k >= parts * TILE64_MIN_SHARE:

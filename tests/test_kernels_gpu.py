@@ -735,7 +735,9 @@ def test_mfma_attention_refuses_what_it_cannot_do():
     (1, 8200, 4096, (0, 0, 0)), (2, 100, 4096, (-1, 8, 16)), (8, 333, 1000, (-1, 16, 4)), (16, 64, 12288, (-1, 4, 8)),
     (11, 50, 72, (-1, 3, 4)), (8, 24576, 512, (-2, 64, 4)), (16, 333, 4096, (-2, 7, 16)), (5, 777, 2000, (-2, 1000, 8)),
     (3, 100, 72, (-2, 3, 4)), (1, 8200, 4096, (-2, 256, 16)), (17, 333, 1000, (-2, 40, 4)), (32, 4096, 2048, (-2, 256, 8)),
-    (25, 50, 1200, (-2, 9, 5)), (40, 333, 1000, (-2, 40, 4)), (64, 200, 1280, (-2, 30, 5)), (49, 77, 1016, (-2, 3, 4)), (8, 200, 4904, (-2, 16, 20))])
+    (25, 50, 1200, (-2, 9, 5)), (40, 333, 1000, (-2, 40, 4)), (64, 200, 1280, (-2, 30, 5)), (49, 77, 1016, (-2, 3, 4)), (8, 200, 4904, (-2, 16, 20)),
+    # 17..32 rows with 12 or 16 pieces a wave: W goes through four slots
+    (24, 777, 4096, (-2, 20, 16)), (32, 300, 4000, (-2, 5, 16)), (17, 200, 3072, (-2, 3, 12)), (30, 64, 2904, (-2, 100, 12))])
 def test_gemm_skinny(m, n, k, shape, out_dtype):
     x = randn(m, k, dtype=torch.bfloat16, seed=30, scale=0.5)
     w = randn(n, k, dtype=torch.bfloat16, seed=31, scale=0.5)
@@ -759,7 +761,8 @@ def test_gemm_skinny(m, n, k, shape, out_dtype):
                                                 (3, 48, 1000, (-1, 2, 2), 4), (8, 4096, 4096, (-2, 512, 4), 4),
                                                 (16, 130, 3000, (-2, 10, 4), 3), (2, 64, 12288, (-2, 30, 16), 3),
                                                 (32, 4096, 4096, (-2, 256, 4), 4), (20, 136, 5120, (-2, 33, 5), 4),
-                                                (64, 520, 4096, (-2, 256, 4), 4), (41, 136, 4800, (-2, 7, 5), 4)])
+                                                (64, 520, 4096, (-2, 256, 4), 4), (41, 136, 4800, (-2, 7, 5), 4),
+                                                (24, 136, 12288, (-2, 4, 16), 3), (32, 100, 9000, (-2, 3, 12), 3)])
 def test_gemm_skinny_shares_out_the_inner_size(m, n, k, shape, ksplit):
     """Partial products [ksplit, M, N] in float: part s covers its own columns only, and the
     ordered sum is the product."""
@@ -949,7 +952,9 @@ def test_linear_follows_its_plan_and_all_roads_agree():
     torch.testing.assert_close(kern.linear(x, narrow).double(), ref, rtol=2e-2, atol=5e-2)
     g, u = wide[0::2].double(), wide[1::2].double()
     ref_act = torch.nn.functional.silu(x.double() @ g.T) * (x.double() @ u.T)
-    for rows in (8, 40):                                                    # staying blocks; library + silu kernel
+    assert kern.streaming_plan(24, 16640, 4096, gate_pairs=True, device=x.device)[0] == (-2, kern.compute_units(x.device), 16)
+    assert kern.streaming_plan(40, 16640, 4096, gate_pairs=True, device=x.device) is None
+    for rows in (8, 24, 40):                    # staying blocks; the same with two row tiles of x; library + activation kernel
         xi = x if rows == 8 else randn(rows, 4096, dtype=torch.bfloat16, seed=39, scale=0.5)
         want = ref_act if rows == 8 else torch.nn.functional.silu(xi.double() @ g.T) * (xi.double() @ u.T)
         got = kern.linear(xi, wide, gate_pairs="silu")
@@ -959,7 +964,8 @@ def test_linear_follows_its_plan_and_all_roads_agree():
 
 @pytest.mark.parametrize("m,inter,k,shape", [(1, 176, 80, (0, 0, 0)), (8, 12288, 96, (0, 0, 0)), (40, 224, 104, (0, 0, 0)),
                                              (16, 1000, 4096, (0, 0, 0)), (8, 1000, 4096, (-2, 256, 16)),
-                                             (3, 177, 1000, (-2, 5, 4))])
+                                             (3, 177, 1000, (-2, 5, 4)), (24, 1000, 4096, (-2, 256, 16)),
+                                             (32, 177, 3000, (-2, 5, 12))])
 @pytest.mark.parametrize("act", ACTIVATIONS)
 def test_gemm_skinny_activation_epilogue(m, inter, k, shape, act):
     """Rows of w alternate gate and up rows; the product comes out as act(gate) * up."""

@@ -7,7 +7,7 @@ import pytest
 
 from jax_vllm_amd.ops import kernels as K
 
-ROWS = [1, 2, 3, 8, 9, 16, 17, 33, 64, 65, 200]
+ROWS = [1, 2, 3, 8, 9, 16, 17, 32, 33, 64, 65, 200]
 WIDTHS = [16, 64, 520, 1024, 2048, 2560, 4096, 5120, 6144, 7168, 8192, 8200, 10240, 24576, 34816, 51200, 151936]
 INNER = [8, 256, 264, 512, 1000, 1024, 1536, 2048, 2560, 3072, 4096, 5120, 6152, 8192, 9728, 12288, 17408, 25600]
 
@@ -26,7 +26,7 @@ def acceptable(m, n, k, silu, plan):
         return "more than 64 rows"
     kind, a, b = shape
     if kind == -2:
-        if (m > 16 and b > 8) or (m > 32 and b > 5) or b not in K.STAY_PIECES or a < 1 or \
+        if (16 < m <= 32 and b not in K.STAY_PIECES_32_ROWS) or (m > 32 and b > 5) or b not in K.STAY_PIECES or a < 1 or \
                 not (256 * b * (parts - 1) < k <= 256 * b * parts):
             return "staying blocks that do not cover the inner size"
     elif kind == -1:
@@ -58,6 +58,10 @@ def test_plans_at_the_sizes_they_were_measured_at():
     assert plan(8, 4096, 12288, partial_ok=True) == ((-2, 256, 12), 4)          # down_proj, 8B
     assert plan(8, 24576, 4096, gate_pairs=True) == ((-2, 256, 16), 1)          # gate and up, 8B
     assert plan(64, 4096, 12288, partial_ok=True) == (K.TILE64, 4)              # down_proj at 64 rows
+    assert plan(24, 24576, 4096, gate_pairs=True) == ((-2, 256, 16), 1)         # gate and up at 17..32 rows: W in slots
+    assert plan(32, 151936, 4096) == ((-2, 256, 16), 1)                         # the output embedding likewise
+    assert plan(33, 24576, 4096, gate_pairs=True) is None                       # beyond: the library
+    assert plan(24, 34816, 5120, gate_pairs=True) is None                       # 20 pieces a wave do not fit beside two row tiles
     assert plan(64, 5120, 17408, partial_ok=True) == (K.TILE64, 3)              # 80 tiles of 64 rows: 3 groups fill 256 units
     assert plan(64, 4096, 4096, partial_ok=True) == ((-2, 256, 4), 4)           # four row tiles of x in registers
     assert plan(64, 5120, 8192, partial_ok=True) is None                        # 8 pieces a wave: too many registers for that
