@@ -227,6 +227,7 @@ def main():
             "seq_len": PROMPT_LEN, "max_context": MAX_CONTEXT, "mean_decode_context": round(mean_ctx, 1),
             "page_size": block, "parallelism": "single-gpu", "rope_theta": cfg["rope_theta"],
             "hip_graphs": bool(llm.config.use_hip_graphs),
+            "decode_ahead": bool(llm.config.decode_ahead),
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

@@ -36,6 +36,7 @@ class EngineConfig:
     max_chunk: Optional[int] = None      # largest prompt portion of one request in one step; None: the budget
     enable_prefix_cache: bool = True     # reuse full pages of equal prompt prefixes
     use_hip_graphs: bool = True          # replay captured decode-only steps
+    decode_ahead: bool = True            # start the decode step after a captured one before its tokens reach the host
     seed: int = 0                        # default sampling seed
 
     def __post_init__(self):

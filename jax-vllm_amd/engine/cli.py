@@ -33,6 +33,8 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--max-chunk", type=int, default=None, help="largest prompt portion of one request per step")
     p.add_argument("--no-prefix-cache", dest="prefix_cache", action="store_false")
     p.add_argument("--no-hip-graphs", dest="hip_graphs", action="store_false")
+    p.add_argument("--no-decode-ahead", dest="decode_ahead", action="store_false",
+                   help="Wait for a decode step's tokens before the next step is started.")
     p.add_argument("--no-prewarm", dest="prewarm", action="store_false",
                    help="Skip building the kernels and capturing the decode steps before the first prompt.")
     p.add_argument("--prompt-ids", action="append", default=[], metavar="'ID ID ...'",
@@ -91,7 +93,8 @@ def main(argv=None) -> int:
               num_blocks=args.num_blocks, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
               max_prefill_len=min(args.max_prefill_len, args.max_model_len),
               max_num_batched_tokens=args.max_num_batched_tokens, max_chunk=args.max_chunk,
-              enable_prefix_cache=args.prefix_cache, use_hip_graphs=args.hip_graphs, seed=args.seed)
+              enable_prefix_cache=args.prefix_cache, use_hip_graphs=args.hip_graphs, decode_ahead=args.decode_ahead,
+              seed=args.seed)
     if args.prewarm:
         print(f"prewarmed in {llm.prewarm():.2f}s", file=sys.stderr, flush=True)
     sp = SamplingParams(max_new_tokens=args.max_new_tokens, eos_id=args.eos_id, temperature=args.temperature)

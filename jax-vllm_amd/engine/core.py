@@ -124,6 +124,7 @@ class EngineCore:
         self._replayable = model.replayable()
         self._spare_slot = config.max_num_seqs     # the state row of rows that pad a captured step
         self.graph_replays = 0
+        self.steps_followed = 0              # decode steps started before the tokens of the step before were on the host
 
     # ---- requests
     def start_request(self, request_id, prompt: Optional[Sequence[int]] = None) -> int:
@@ -172,17 +173,52 @@ class EngineCore:
             return False
         return all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)
 
-    def _run_decode_graph(self, entries) -> torch.Tensor:
+    def _graph_key(self, request_ids, more_tokens: int = 0) -> tuple:
+        """(rows, block-table widths) of the captured step that serves these requests, once each of
+        them has pages for ``more_tokens`` further tokens."""
+        cache = self.cache
+        have = [[len(cache.block_table(r, g)) + (cache.pages_needed(r, more_tokens)[g] if more_tokens else 0)
+                 for r in request_ids] for g in range(len(self.group_keys))]
+        return _batch_bucket(len(request_ids)), tuple(_bucket(max(h), 8) for h in have)
+
+    def follow_decode(self, request_ids: Sequence, token_source: torch.Tensor) -> Optional[torch.Tensor]:
+        """One more decode step of exactly these requests (each has one token's logits on the way),
+        launched before the tokens are known on the host: row i takes its token from
+        ``token_source[i]`` (int32, on the device, written by work already on the stream).  Only a
+        step that is already captured and whose pages are free is launched; otherwise None, and
+        nothing has changed.  The caller commits each request's token (``commit_decode``) once it
+        knows it, before anything else is asked of that request."""
+        if not self.config.use_hip_graphs or not self._replayable or not 0 < len(request_ids) <= self._max_graph_batch:
+            return None
+        cache = self.cache
+        g = self._graphs.get(self._graph_key(request_ids, 1))
+        if g is None or g.graph is None:
+            return None
+        promised = [0] * len(self.group_keys)
+        for r in request_ids:
+            if not cache.can_store(r, 1, reserve=promised):
+                return None
+            promised = [p + n for p, n in zip(promised, cache.pages_needed(r, 1))]
+        for r in request_ids:
+            cache.reserve(r, 1)
+        self.steps_followed += 1
+        return self._run_decode_graph([StepEntry(r, [0], [0]) for r in request_ids], token_source)
+
+    def commit_decode(self, request_id, token: int) -> None:
+        """The token that a step of ``follow_decode`` read for this request from the device."""
+        self.cache.commit(request_id, [int(token)])
+
+    def _run_decode_graph(self, entries, token_source: Optional[torch.Tensor] = None) -> torch.Tensor:
         """A step of single tokens, one per request, each wanting its logits: the launch sequence
         is captured once per (batch bucket, table-width bucket) and replayed from fixed buffers;
-        rows added to reach the bucket size read the null page and store nothing."""
+        rows added to reach the bucket size read the null page and store nothing.  With
+        ``token_source`` the tokens are copied from there on the device instead of coming from the
+        entries."""
         cache, ps = self.cache, self.page_size
         r = len(entries)
-        rb = _batch_bucket(r)
         n_groups = len(self.group_keys)
-        widths = tuple(_bucket(max(len(cache.block_table(e.request_id, g)) for e in entries), 8)
-                       for g in range(n_groups))
-        key = (rb, widths)
+        key = self._graph_key([e.request_id for e in entries])
+        rb, widths = key
         g = self._graphs.get(key)
         if g is None:
             g = self._graphs[key] = _DecodeGraph(rb, widths, n_groups, self.device)
@@ -221,6 +257,8 @@ class EngineCore:
         if g.copied is None:
             g.copied = torch.cuda.Event()
         g.copied.record()
+        if token_source is not None:
+            g.dev_segment("tokens")[:r].copy_(token_source[:r])
         if g.graph is None:
             # first use: run the launches eagerly (this is the step's result), then record them
             ctx = g.context(ps, self.page_size * max(widths, default=1))

@@ -18,17 +18,37 @@ from .request import EngineStats, Request, SamplingParams, StepEvent
 from .scheduler import Scheduler
 
 
+class _StepUnderWay:
+    """A decode step that is already on the GPU: its items, and its tokens being chosen."""
+
+    def __init__(self, items: list, drawn):
+        self.items, self.drawn = items, drawn
+
+
 class Engine:
     """The host loop above the step function: requests in, ``StepEvent``s out.  It needs a cache
     manager for the scheduler, a ``run(entries, borrow=True)`` that returns logits for the
     wanted places, and a ``sample(logits, temperatures, keys)``; the GPU engine passes the real
-    ones, host-only tests pass stand-ins."""
+    ones, host-only tests pass stand-ins.
 
-    def __init__(self, config: EngineConfig, cache, run, sample, vocab_size: int):
+    ``ahead`` (optional; the GPU engine passes one): lets a decode step follow the one before it
+    on the GPU without the host in between.  It has ``launch(logits, temperatures, keys)`` and
+    ``finish(drawn)``, the two halves of ``sample``; ``follow(request_ids, drawn)``, which starts
+    one more decode step of the same requests with each row's token taken from the device, or
+    returns None; and ``commit(request_id, token)`` for the tokens of such a step once they are
+    known.  While step k runs, ``step`` then already starts step k + 1 of the same requests,
+    waits for the tokens of step k only afterwards and returns step k's events as ever; the
+    next call finds its step under way.  Only a step of decodes of every running request is
+    followed, with nobody waiting, none of them at its last token and pages at hand; a request
+    that ends on its ``eos_id`` has one row of the step under way for nothing, which is ignored."""
+
+    def __init__(self, config: EngineConfig, cache, run, sample, vocab_size: int, ahead=None):
         self.config = config
         self.stats = EngineStats()
         self.scheduler = Scheduler(config, cache, self.stats)
         self._run, self._sample = run, sample
+        self._ahead = ahead
+        self._under_way: Optional[_StepUnderWay] = None
         self.vocab_size = vocab_size
         self._next_id = 0
         self.requests: dict = {}     # waiting and running requests by id; a finished one leaves with its last event
@@ -52,42 +72,79 @@ class Engine:
     def has_work(self) -> bool:
         return self.scheduler.has_work()
 
-    def step(self) -> list:
-        """One scheduler iteration: schedule, run the mixed batch, sample, finish.  Returns the
-        ``StepEvent`` of every token emitted.  The event that finishes a request carries the
-        request (prompt, output, counters); the engine keeps nothing of it afterwards."""
-        out = self.scheduler.schedule()
-        if not out.items:
-            return []
-        entries, sampled = [], []
-        for item in out.items:
-            req = item.request
-            tokens = req.all_tokens[req.num_computed:req.num_computed + item.num_tokens]
-            entries.append(StepEntry(req.request_id, tokens, [item.num_tokens - 1] if item.samples else []))
-            if item.samples:
-                sampled.append(item)
-            if item.num_tokens == 1 and item.samples and req.output_ids:
+    def _draw_arguments(self, sampled: list, ahead_by: int = 0):
+        temps = [i.request.sampling.temperature for i in sampled]
+        keys = [
+            draw_key(i.request.sampling.seed if i.request.sampling.seed is not None else self.config.seed,
+                     i.request.request_id, len(i.request.output_ids) + ahead_by)
+            for i in sampled
+        ]
+        return temps, keys
+
+    def _count(self, items: list) -> None:
+        for item in items:
+            if item.num_tokens == 1 and item.samples and item.request.output_ids:
                 self.stats.decode_tokens += 1
                 self.stats.decode_calls += 1
             else:
                 self.stats.prefill_tokens += item.num_tokens
                 self.stats.prefill_portions += 1
         self.stats.steps_run += 1
-        self.stats.max_batched_tokens = max(self.stats.max_batched_tokens, out.num_tokens)
-        logits = self._run(entries, borrow=True)
-        temps = [i.request.sampling.temperature for i in sampled]
-        keys = [
-            draw_key(i.request.sampling.seed if i.request.sampling.seed is not None else self.config.seed,
-                     i.request.request_id, len(i.request.output_ids))
-            for i in sampled
-        ]
-        tokens = self._sample(logits, temps, keys)
-        events, k = [], 0
-        for item in out.items:
-            tok = None
-            if item.samples:
-                tok = tokens[k]
-                k += 1
+        self.stats.max_batched_tokens = max(self.stats.max_batched_tokens, sum(i.num_tokens for i in items))
+
+    def _may_follow(self, items: list) -> bool:
+        """Whether the step after this one is known already: the same decodes again."""
+        sch = self.scheduler
+        if self._ahead is None or sch.waiting or len(items) != len(sch.running):
+            return False
+        return all(i.num_tokens == 1 and i.samples and i.request.output_ids
+                   and len(i.request.output_ids) + 1 < i.request.sampling.max_new_tokens for i in items)
+
+    def step(self) -> list:
+        """One scheduler iteration: schedule, run the mixed batch, sample, finish.  Returns the
+        ``StepEvent`` of every token emitted.  The event that finishes a request carries the
+        request (prompt, output, counters); the engine keeps nothing of it afterwards."""
+        under_way, self._under_way = self._under_way, None
+        tokens = drawn = None
+        if under_way is not None and any(not i.request.finished for i in under_way.items):
+            # the step that the call before this one started: row k belongs to its k-th item; the rows of
+            # requests that ended on their eos_id meanwhile are not looked at
+            row_of = {id(i): k for k, i in enumerate(under_way.items)}
+            items = [i for i in under_way.items if not i.request.finished]
+            drawn = under_way.drawn
+            self.scheduler.step_index += 1
+        else:
+            out = self.scheduler.schedule()
+            if not out.items:
+                return []
+            items = out.items
+            entries = []
+            for item in items:
+                req = item.request
+                toks = req.all_tokens[req.num_computed:req.num_computed + item.num_tokens]
+                entries.append(StepEntry(req.request_id, toks, [item.num_tokens - 1] if item.samples else []))
+            logits = self._run(entries, borrow=True)
+            sampled = [i for i in items if i.samples]
+            row_of = {id(i): k for k, i in enumerate(sampled)}
+            temps, keys = self._draw_arguments(sampled)
+            if self._ahead is not None and sampled:
+                drawn = self._ahead.launch(logits, temps, keys)
+            else:
+                tokens = self._sample(logits, temps, keys)
+        self._count(items)
+        # the step after this one, if it is known already, goes to the GPU before this one's tokens are awaited
+        following = None
+        if drawn is not None and [row_of.get(id(i)) for i in items] == list(range(drawn.rows)) and self._may_follow(items):
+            logits = self._ahead.follow([i.request.request_id for i in items], drawn)
+            if logits is not None:
+                nxt = [type(i)(i.request, 1, True) for i in items]
+                temps, keys = self._draw_arguments(nxt, ahead_by=1)
+                following = _StepUnderWay(nxt, self._ahead.launch(logits, temps, keys))
+        if drawn is not None:
+            tokens = self._ahead.finish(drawn)
+        events = []
+        for item in items:
+            tok = tokens[row_of[id(item)]] if item.samples else None
             finished = self.scheduler.advance(item, tok)
             if tok is not None:
                 self.stats.emitted_tokens += 1
@@ -95,10 +152,16 @@ class Engine:
                                         item.request if finished else None))
             if finished:
                 self.requests.pop(item.request.request_id, None)
+        if following is not None:
+            for item in following.items:     # the step under way has read these tokens from the device
+                if not item.request.finished:
+                    self._ahead.commit(item.request.request_id, item.request.output_ids[-1])
+            self._under_way = following
         return events
 
     def abort_all(self) -> None:
         """Drop every waiting and running request and give back what they hold."""
+        self._under_way = None             # what it has on the GPU ends by itself and is never looked at
         self.scheduler.waiting.clear()
         for req in list(self.scheduler.running):
             self.scheduler.finish(req)
@@ -116,6 +179,17 @@ class Engine:
         while self.has_work():
             self.step()
         return [list(r.output_ids) for r in reqs]
+
+
+class _Ahead:
+    """What ``Engine`` needs to let a decode step follow the one before it on the GPU."""
+
+    def __init__(self, core, sampler):
+        self.core, self.launch, self.finish = core, sampler.launch, sampler.finish
+        self.commit = core.commit_decode
+
+    def follow(self, request_ids, drawn):
+        return self.core.follow_decode(request_ids, drawn.tokens)
 
 
 class LLM(Engine):
@@ -143,7 +217,8 @@ class LLM(Engine):
             self.model, self.model_config = load_model(Path(model), config.dtype, device)
         self.core = EngineCore(self.model, config)
         self.sampler = Sampler(self.core.device)
-        super().__init__(config, self.core.cache, self.core.run, self.sampler.sample, self.core.vocab_size)
+        super().__init__(config, self.core.cache, self.core.run, self.sampler.sample, self.core.vocab_size,
+                         ahead=_Ahead(self.core, self.sampler) if config.decode_ahead else None)
         self._replays_before = 0     # replays of a prewarm are not the requests'
 
     def step(self) -> list:

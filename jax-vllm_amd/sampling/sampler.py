@@ -16,25 +16,58 @@ from ..ops import kernels as K
 from .keys import draw_key  # noqa: F401  (re-exported)
 
 
+class Drawn:
+    """Tokens that the GPU is still choosing: ``tokens`` on the device (int32, one per row), their copy to
+    pinned host memory under way, and the event after that copy."""
+
+    def __init__(self, tokens: torch.Tensor, host: torch.Tensor, copied, rows: int, vocab: int):
+        self.tokens, self.host, self.copied, self.rows, self.vocab = tokens, host, copied, rows, vocab
+
+
 class Sampler:
+    HOST_BUFFERS = 4          # pinned buffers in turn: more than the steps that are ever under way at once
+
     def __init__(self, device):
         self.device = device
+        self._host, self._turn = [], 0
 
-    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], keys: Sequence[int]) -> list:
-        """One token id per row of ``logits`` [M, V] (float32, on the device)."""
+    def _pinned(self, rows: int) -> torch.Tensor:
+        if len(self._host) < self.HOST_BUFFERS:
+            self._host.append(torch.empty(max(rows, 64), dtype=torch.int32, pin_memory=True))
+        self._turn = (self._turn + 1) % len(self._host)
+        if self._host[self._turn].numel() < rows:
+            self._host[self._turn] = torch.empty(rows, dtype=torch.int32, pin_memory=True)
+        return self._host[self._turn]
+
+    def launch(self, logits: torch.Tensor, temperatures: Sequence[float], keys: Sequence[int]) -> Drawn:
+        """Start choosing one token id per row of ``logits`` [M, V] (float32, on the device) and copying
+        them to the host; nothing here waits for the GPU."""
         m = logits.shape[0]
-        if m == 0:
-            return []
         if all(t <= 0.0 for t in temperatures):
             out = K.sample(logits)
         else:
             temp = torch.tensor(list(temperatures), dtype=torch.float32, device=self.device)
             key = torch.tensor(list(keys), dtype=torch.int64, device=self.device)
             out = K.sample(logits, temp, key)
-        ids = out.tolist()
-        vocab = logits.shape[1]
-        bad = [i for i, t in enumerate(ids) if not 0 <= t < vocab]
+        host = self._pinned(m)
+        host[:m].copy_(out, non_blocking=True)
+        copied = torch.cuda.Event()
+        copied.record()
+        return Drawn(out, host, copied, m, logits.shape[1])
+
+    def finish(self, drawn: Drawn) -> list:
+        """The token ids of a ``launch``, once they are there."""
+        drawn.copied.synchronize()
+        ids = drawn.host[:drawn.rows].tolist()
+        bad = [i for i, t in enumerate(ids) if not 0 <= t < drawn.vocab]
         if bad:
             # the kernel answers "no token" (the vocabulary size) for a row without any comparable value
-            raise FloatingPointError(f"logits row(s) {bad} of {m} hold no finite maximum (NaN): no token can be chosen")
+            raise FloatingPointError(
+                f"logits row(s) {bad} of {drawn.rows} hold no finite maximum (NaN): no token can be chosen")
         return ids
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], keys: Sequence[int]) -> list:
+        """One token id per row of ``logits`` [M, V] (float32, on the device)."""
+        if logits.shape[0] == 0:
+            return []
+        return self.finish(self.launch(logits, temperatures, keys))

@@ -265,6 +265,55 @@ def test_replayed_decode_steps_equal_eager_steps(folders, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_decode_steps_started_ahead_give_the_same_tokens(folders, dtype):
+    """With ``decode_ahead`` a captured decode step is started before the tokens of the step before
+    it are on the host (it takes them from the sampling output on the device).  Greedy and drawn
+    tokens, requests that end on an eos_id in the middle of that (one row of the step under way is
+    then for nothing), requests that join later and prefixes taken from the cache: the tokens are
+    those of an engine that waits for every step, and those of the plain implementation."""
+    from jax_vllm_amd import LLM, SamplingParams
+
+    cfg, w = plain_of(folders["B"])
+    rng = np.random.default_rng(17)
+    shared = rng.integers(0, cfg["vocab_size"], size=40).tolist()
+    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (9, 33, 18)] + [shared + [3, 4], shared + [5]]
+    plain = [P.greedy_generate(w, cfg, p, 24) for p in prompts]
+    params = [SamplingParams(max_new_tokens=24), SamplingParams(max_new_tokens=24, eos_id=plain[1][7]),
+              SamplingParams(max_new_tokens=17, temperature=0.8, seed=5), SamplingParams(max_new_tokens=24),
+              SamplingParams(max_new_tokens=20, eos_id=plain[4][11])]
+    outs = {}
+    for ahead in (False, True):
+        llm = LLM(folders["B"], dtype=dtype, block_size=16, max_num_seqs=5, max_model_len=128,
+                  max_num_batched_tokens=64, decode_ahead=ahead)
+        got = {}
+        rids = [llm.add_request(p, sp) for p, sp in zip(prompts[:3], params[:3])]
+        calls = 0
+        while llm.has_work():
+            for ev in llm.step():
+                got.setdefault(ev.request_id, []).append(ev.token)
+            calls += 1
+            if calls in (6, 13):          # two requests join while decode steps follow each other
+                rids.append(llm.add_request(prompts[len(rids)], params[len(rids)]))
+        outs[ahead] = [got[r] for r in rids]
+        assert (llm.core.steps_followed > 10) == ahead and llm.core.graph_replays > 10
+        llm.core.cache.check_invariants()
+        assert llm.core.cache.num_free_pages() == llm.config.usable_pages and not llm.core.cache.requests
+        assert llm.stats.cache_hit_tokens >= 32
+        again = llm.generate(prompts[:2], params[:2])             # the engine is as good as new afterwards
+        assert again == outs[ahead][:2]
+    assert outs[True] == outs[False]
+    for i in (0, 1, 3, 4):                                        # the greedy ones against the plain implementation
+        got = outs[True][i]
+        eos = params[i].eos_id
+        if dtype == "float32":
+            want = plain[i][:plain[i].index(eos) + 1] if eos is not None and eos in plain[i] else plain[i][:params[i].max_new_tokens]
+            assert got == want
+        else:
+            check_tokens_follow(dtype, cfg, w, prompts[i], got)
+    assert len(outs[True][2]) == 17
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_replayed_decode_steps_of_many_requests(folders, dtype):
     """Captured decode steps with 20 and then 40 live requests (rows of the step: 24 and 48, of
     which the last are padding), while requests end and the rows are handed to others: every

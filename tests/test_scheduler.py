@@ -300,3 +300,153 @@ def test_the_stepped_loop_hands_out_finished_requests_and_keeps_none():
         assert tokens[rid] == done[rid].output_ids == expected(p, 5 + i) and done[rid].prompt_ids == p
     core.cache.check_invariants()
     assert core.cache.num_free_pages() == eng.config.usable_pages
+
+
+# ------------------------------------------------------------------ a decode step started ahead of the tokens
+class FakeDrawn:
+    def __init__(self, tokens):
+        self.tokens, self.rows = list(tokens), len(tokens)
+
+
+class FakeAhead:
+    """What the GPU engine hands the loop so that a decode step can follow the one before it: here
+    on the host, with the same duties towards the cache manager (pages reserved at the start of the
+    step, the token committed once the loop knows it)."""
+
+    def __init__(self, core, refuse_every=0):
+        self.core, self.refuse_every = core, refuse_every
+        self.asked = self.followed = 0
+        self.committed = []
+
+    @staticmethod
+    def launch(rows, temps, keys):
+        assert len(rows) == len(temps) == len(keys)
+        return FakeDrawn(rows)
+
+    @staticmethod
+    def finish(drawn):
+        return drawn.tokens
+
+    def follow(self, request_ids, drawn):
+        cache = self.core.cache
+        self.asked += 1
+        if self.refuse_every and self.asked % self.refuse_every == 0:
+            return None                                  # as if that step had not been captured yet
+        promised = [0] * len(cache.groups)
+        for r in request_ids:
+            if not cache.can_store(r, 1, reserve=promised):
+                return None
+            promised = [p + n for p, n in zip(promised, cache.pages_needed(r, 1))]
+        rows, log = [], []
+        for k, r in enumerate(request_ids):
+            cache.reserve(r, 1)
+            ctx = cache.requests[r].tokens
+            log.append((r, len(ctx), 1, [0]))
+            rows.append(next_token(ctx + [drawn.tokens[k]]))
+        self.core.steps.append(log)
+        self.followed += 1
+        return rows
+
+    def commit(self, request_id, token):
+        self.committed.append((request_id, token))
+        self.core.cache.commit(request_id, [token])
+        self.core.cache.check_invariants()
+
+
+def make_ahead(refuse_every=0, **kw):
+    cfg = EngineConfig(**kw)
+    core = FakeCore(cfg)
+    ahead = FakeAhead(core, refuse_every)
+    return Engine(cfg, core.cache, core.run, core.sample, VOCAB, ahead=ahead), core, ahead
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_steps_started_ahead_change_nothing_that_a_caller_sees(seed):
+    """The same requests through the loop with and without decode steps started ahead: the events
+    of every call of ``step`` are the same (a step started ahead may hold a row more, of a request
+    that ended on its eos_id in the step before)."""
+    rng = np.random.default_rng(100 + seed)
+    n = 7
+    prompts = [rng.integers(0, 5, size=int(rng.integers(1, 30))).tolist() for _ in range(n)]
+    params = [SamplingParams(max_new_tokens=int(rng.integers(1, 24)), eos_id=int(rng.integers(0, VOCAB)) if i % 2 else None)
+              for i in range(n)]
+    kw = dict(block_size=4, max_num_seqs=n if seed % 2 else int(rng.integers(2, 6)), max_model_len=64,
+              max_num_batched_tokens=int(rng.integers(8, 40)), num_blocks=1 + int(rng.integers(20, 40)))
+    logs = []
+    for refuse in (None, 0, 3):
+        if refuse is None:
+            eng, core = make(**kw)
+            ahead = None
+        else:
+            eng, core, ahead = make_ahead(refuse, **kw)
+        for p, sp in zip(prompts, params):
+            eng.add_request(p, sp)
+        events = [[(e.request_id, e.token, e.finished) for e in step] for step in drain(eng)]
+        core.cache.check_invariants()
+        assert core.cache.num_free_pages() == eng.config.usable_pages and not core.cache.requests
+        logs.append((events, eng.stats.emitted_tokens, eng.stats.decode_tokens, eng.stats.steps_run))
+        if ahead is not None and seed % 2:              # with a slot for everybody nobody waits: steps do follow
+            assert ahead.followed > 0
+    assert logs[0] == logs[1] == logs[2]
+
+
+def test_a_step_is_started_ahead_only_when_the_next_one_is_known():
+    eng, core, ahead = make_ahead(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=32)
+    a = eng.add_request([1, 2, 3], SamplingParams(max_new_tokens=4))
+    b = eng.add_request([4, 5], SamplingParams(max_new_tokens=6))
+    c = eng.add_request([6], SamplingParams(max_new_tokens=5))           # waits for a slot
+    eng.step()                                                            # prompts of a and b: nothing to follow
+    assert ahead.asked == 0 and eng._under_way is None
+    eng.step()                                                            # decodes, but c waits: the next step is not known
+    eng.step()
+    assert ahead.asked == 0
+    eng.step()                                                            # a ends here (4 tokens): c is admitted next
+    assert a not in eng.requests and ahead.asked == 0
+    eng.step()                                                            # b decodes beside c's prompt
+    assert ahead.asked == 0
+    eng.step()                                                            # b's last token: not followed either
+    assert b not in eng.requests and ahead.asked == 0
+    eng.step()                                                            # c alone, its third token of five: followed
+    assert ahead.asked == 1 and eng._under_way is not None
+    events = eng.step()                                                   # the step under way, and one more after it
+    assert [(e.request_id, e.finished) for e in events] == [(c, False)] and ahead.asked == 2
+    events = eng.step()                                                   # c's last token: nothing follows
+    assert [(e.request_id, e.finished) for e in events] == [(c, True)] and ahead.asked == 2
+    assert not eng.has_work() and eng._under_way is None
+    assert core.cache.num_free_pages() == eng.config.usable_pages
+    assert events[0].request.output_ids == expected([6], 5)
+
+
+def test_a_request_that_ends_on_its_eos_leaves_a_row_of_the_step_under_way_unused():
+    prompts = [[1, 2, 3], [4, 5, 6, 7]]
+    want = [expected(p, 12) for p in prompts]
+    eos = want[0][3]                                  # the first request ends with its 4th token ...
+    assert eos not in want[0][:3], "pick another prompt"
+    eng, core, ahead = make_ahead(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=32)
+    a = eng.add_request(prompts[0], SamplingParams(max_new_tokens=12, eos_id=eos))
+    b = eng.add_request(prompts[1], SamplingParams(max_new_tokens=12))
+    out = {a: [], b: []}
+    ended_at = None
+    for call in range(40):
+        if not eng.has_work():
+            break
+        for e in eng.step():
+            out[e.request_id].append(e.token)
+            if e.request_id == a and e.finished:
+                ended_at = call
+                assert eng._under_way is not None     # ... while the step after it was already started with a row for it
+                assert [i.request.request_id for i in eng._under_way.items] == [a, b]
+    assert out[a] == want[0][:4] and out[b] == want[1] and ended_at is not None
+    assert all(r != a or t != eos for r, t in ahead.committed)           # its last token was never committed: it had ended
+    assert core.cache.num_free_pages() == eng.config.usable_pages and not core.cache.requests
+
+
+def test_abort_with_a_step_under_way():
+    eng, core, ahead = make_ahead(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=32)
+    eng.add_request([1, 2, 3], SamplingParams(max_new_tokens=10))
+    eng.step(), eng.step()
+    assert eng._under_way is not None
+    eng.abort_all()
+    assert eng._under_way is None and not eng.has_work()
+    assert core.cache.num_free_pages() == eng.config.usable_pages
+    assert eng.generate([[5, 6]], SamplingParams(max_new_tokens=5)) == [expected([5, 6], 5)]
