@@ -15,7 +15,7 @@ from ..config.engine import EngineConfig
 from ..sampling.keys import draw_key
 from .entries import StepEntry
 from .request import EngineStats, Request, SamplingParams, StepEvent
-from .scheduler import Scheduler
+from .scheduler import ScheduledItem, Scheduler
 
 
 class _StepUnderWay:
@@ -137,7 +137,7 @@ class Engine:
         if drawn is not None and [row_of.get(id(i)) for i in items] == list(range(drawn.rows)) and self._may_follow(items):
             logits = self._ahead.follow([i.request.request_id for i in items], drawn)
             if logits is not None:
-                nxt = [type(i)(i.request, 1, True) for i in items]
+                nxt = [ScheduledItem(i.request, 1, True) for i in items]
                 temps, keys = self._draw_arguments(nxt, ahead_by=1)
                 following = _StepUnderWay(nxt, self._ahead.launch(logits, temps, keys))
         if drawn is not None:
