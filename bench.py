@@ -100,6 +100,29 @@ def measure_prefill(llm, rng, vocab, repeats=3):
     return best
 
 
+def measure_long_prompt(llm, rng, vocab, prompt_len):
+    """One prompt of ``prompt_len`` tokens through the engine in portions of the token budget, from the
+    request's arrival to its first token (a short prompt first, untimed, so that nothing is set up
+    inside the timed part)."""
+    from jax_vllm_amd import SamplingParams
+
+    one = SamplingParams(max_new_tokens=1)
+    llm.generate([rng.integers(0, vocab, size=llm.config.max_num_batched_tokens).tolist()], one)
+    sync()
+    prompt = rng.integers(0, vocab, size=prompt_len).tolist()
+    t0 = time.perf_counter()
+    llm.add_request(prompt, one)
+    steps, last = 0, 0.0
+    while llm.has_work():
+        t1 = time.perf_counter()
+        llm.step()
+        sync()
+        last, steps = time.perf_counter() - t1, steps + 1
+    dt = time.perf_counter() - t0
+    return {"prompt_tokens_per_s": round(prompt_len / dt, 1), "seconds": round(dt, 4), "prompt_len": prompt_len,
+            "portions": steps, "last_portion_ms": round(last * 1e3, 3)}
+
+
 def measure_mixed(llm, rng, vocab, running=32, joining=4, join_len=3000, shared=1024):
     """A continuous-batching mix: ``running`` requests decode at contexts
     uniform in [512, 4096] when ``joining`` prompts of ``join_len`` tokens arrive, two of which share
@@ -146,13 +169,17 @@ def main():
                     help="run only the first layers of the shape's (both numbers are reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="measure the headline batch only")
-    ap.add_argument("--only", choices=["prefill", "decode", "mixed"], default=None,
+    ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt"], default=None,
                     help="run one phase alone and print its result (for profiling); mixed: 32 running decodes "
-                         "joined by 4 prompts of 3,000 tokens in portions of 512 under a budget of 2,048")
+                         "joined by 4 prompts of 3,000 tokens in portions of 512 under a budget of 2,048; "
+                         "long-prompt: one prompt of --prompt-len tokens (default 32,768) in portions of 2,048")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
-    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
-                    help="with --only decode: prompt length of the decoding requests (long-context runs)")
+    ap.add_argument("--prompt-len", type=int, default=None,
+                    help="with --only decode: prompt length of the decoding requests (long-context runs, default "
+                         "1,024); with --only long-prompt: the prompt's length")
     args = ap.parse_args()
+    if args.prompt_len is None:
+        args.prompt_len = 32768 if args.only == "long-prompt" else PROMPT_LEN
     world = int(os.environ.get("WORLD_SIZE", "1"))
     if args.gpus != 1 or world != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {max(args.gpus, world)} is not supported")
@@ -187,6 +214,11 @@ def main():
     wbytes, per_layer_params = weight_bytes(cfg, layers, itemsize)
     kv_per_token = llm.core.kv_bytes_per_token
 
+    if args.only == "long-prompt":
+        res = measure_long_prompt(llm, rng, vocab, args.prompt_len)
+        res.update(model=model_name, layers=layers)
+        print(json.dumps(res), flush=True)
+        return
     if args.only == "prefill":
         pre_s = measure_prefill(llm, rng, vocab)
         print(json.dumps({"prefill_ms": round(pre_s * 1e3, 3), "tokens": PREFILL_TOKENS, "layers": layers}), flush=True)
