@@ -39,8 +39,9 @@ class Engine:
     known.  While step k runs, ``step`` then already starts step k + 1 of the same requests,
     waits for the tokens of step k only afterwards and returns step k's events as ever; the
     next call finds its step under way.  Only a step of decodes of every running request is
-    followed, with nobody waiting, none of them at its last token and pages at hand; a request
-    that ends on its ``eos_id`` has one row of the step under way for nothing, which is ignored."""
+    followed, with nobody waiting for a free slot, none of them at its last token and pages at
+    hand; a request that ends on its ``eos_id`` has one row of the step under way for nothing,
+    which is ignored (whoever waits for its slot is admitted one step later than otherwise)."""
 
     def __init__(self, config: EngineConfig, cache, run, sample, vocab_size: int, ahead=None):
         self.config = config
@@ -95,8 +96,10 @@ class Engine:
     def _may_follow(self, items: list) -> bool:
         """Whether the step after this one is known already: the same decodes again."""
         sch = self.scheduler
-        if self._ahead is None or sch.waiting or len(items) != len(sch.running):
+        if self._ahead is None or len(items) != len(sch.running):
             return False
+        if sch.waiting and len(sch.running) < self.config.max_num_seqs:
+            return False                     # somebody may be admitted (with every slot taken nobody is)
         return all(i.num_tokens == 1 and i.samples and i.request.output_ids
                    and len(i.request.output_ids) + 1 < i.request.sampling.max_new_tokens for i in items)
 

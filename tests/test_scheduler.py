@@ -384,10 +384,17 @@ def test_steps_started_ahead_change_nothing_that_a_caller_sees(seed):
         events = [[(e.request_id, e.token, e.finished) for e in step] for step in drain(eng)]
         core.cache.check_invariants()
         assert core.cache.num_free_pages() == eng.config.usable_pages and not core.cache.requests
-        logs.append((events, eng.stats.emitted_tokens, eng.stats.decode_tokens, eng.stats.steps_run))
-        if ahead is not None and seed % 2:              # with a slot for everybody nobody waits: steps do follow
+        per_request = {}
+        for step in events:
+            for r, t, _ in step:
+                per_request.setdefault(r, []).append(t)
+        # with a slot for everybody nobody ever waits and every call gives the same events; otherwise a request
+        # that waits for the slot of one that ends on its eos_id is admitted one step later
+        logs.append((per_request, eng.stats.emitted_tokens, events if seed % 2 else None))
+        if ahead is not None and seed % 2:
             assert ahead.followed > 0
     assert logs[0] == logs[1] == logs[2]
+    assert logs[0][0] == {i: expected(p, sp.max_new_tokens, sp.eos_id) for i, (p, sp) in enumerate(zip(prompts, params))}
 
 
 def test_a_step_is_started_ahead_only_when_the_next_one_is_known():
@@ -397,24 +404,32 @@ def test_a_step_is_started_ahead_only_when_the_next_one_is_known():
     c = eng.add_request([6], SamplingParams(max_new_tokens=5))           # waits for a slot
     eng.step()                                                            # prompts of a and b: nothing to follow
     assert ahead.asked == 0 and eng._under_way is None
-    eng.step()                                                            # decodes, but c waits: the next step is not known
-    eng.step()
-    assert ahead.asked == 0
-    eng.step()                                                            # a ends here (4 tokens): c is admitted next
-    assert a not in eng.requests and ahead.asked == 0
-    eng.step()                                                            # b decodes beside c's prompt
-    assert ahead.asked == 0
-    eng.step()                                                            # b's last token: not followed either
-    assert b not in eng.requests and ahead.asked == 0
-    eng.step()                                                            # c alone, its third token of five: followed
+    eng.step()                                                            # decodes; c waits, but every slot is taken: followed
     assert ahead.asked == 1 and eng._under_way is not None
+    eng.step()                                                            # the step under way, and the one after it
+    assert ahead.asked == 2
+    eng.step()                                                            # a's last token (4): the next step is another one
+    assert a not in eng.requests and ahead.asked == 2 and eng._under_way is None
+    eng.step()                                                            # b decodes beside c's prompt
+    assert ahead.asked == 2
+    eng.step()                                                            # b's last token: not followed either
+    assert b not in eng.requests and ahead.asked == 2
+    eng.step()                                                            # c alone, its third token of five: followed
+    assert ahead.asked == 3 and eng._under_way is not None
     events = eng.step()                                                   # the step under way, and one more after it
-    assert [(e.request_id, e.finished) for e in events] == [(c, False)] and ahead.asked == 2
+    assert [(e.request_id, e.finished) for e in events] == [(c, False)] and ahead.asked == 4
     events = eng.step()                                                   # c's last token: nothing follows
-    assert [(e.request_id, e.finished) for e in events] == [(c, True)] and ahead.asked == 2
+    assert [(e.request_id, e.finished) for e in events] == [(c, True)] and ahead.asked == 4
     assert not eng.has_work() and eng._under_way is None
     assert core.cache.num_free_pages() == eng.config.usable_pages
     assert events[0].request.output_ids == expected([6], 5)
+    # a free slot and somebody waiting for it: the next step is not known
+    d = eng.add_request([7, 8], SamplingParams(max_new_tokens=6))
+    eng.step(), eng.step()
+    assert eng._under_way is not None
+    e = eng.add_request([9], SamplingParams(max_new_tokens=2))
+    eng.step()
+    assert eng._under_way is None and d in eng.requests and e in eng.requests
 
 
 def test_a_request_that_ends_on_its_eos_leaves_a_row_of_the_step_under_way_unused():
