@@ -223,10 +223,12 @@ class LLM(Engine):
         super().__init__(config, self.core.cache, self.core.run, self.sampler.sample, self.core.vocab_size,
                          ahead=_Ahead(self.core, self.sampler) if config.decode_ahead else None)
         self._replays_before = 0     # replays of a prewarm are not the requests'
+        self._followed_before = 0
 
     def step(self) -> list:
         events = super().step()
         self.stats.graph_replays = self.core.graph_replays - self._replays_before
+        self.stats.steps_ahead = self.core.steps_followed - self._followed_before
         return events
 
     def prewarm(self) -> float:
@@ -262,6 +264,7 @@ class LLM(Engine):
             self.stats, self._next_id = saved[0], saved[1]
             self.scheduler.stats = self.stats
             self._replays_before = self.core.graph_replays
+            self._followed_before = self.core.steps_followed
         torch.cuda.synchronize()
         return time.perf_counter() - t0
 

@@ -51,7 +51,7 @@ class StepEvent:
 @dataclass
 class EngineStats:
     admissions: int = 0
-    scheduler_loops: int = 0
+    scheduler_loops: int = 0          # decisions of the scheduler (a decode step started ahead of its tokens needs none)
     steps_run: int = 0                # steps that ran at least one token
     prefill_tokens: int = 0           # prompt (or recomputed) tokens run
     decode_tokens: int = 0            # single decoded tokens run
@@ -65,3 +65,4 @@ class EngineStats:
     prefix_waits: int = 0             # admissions put off until a running request had computed shared pages
     max_batched_tokens: int = 0
     graph_replays: int = 0
+    steps_ahead: int = 0              # decode steps started before the tokens of the step before were on the host
