@@ -1,12 +1,10 @@
 """Device side of the cache: page storage for every run that keeps keys and values, state
 rows for every run that keeps state, and the grouping of runs by need.
 
-Key pages are ``[pages + 1, kv_heads, page_size, head_dim]``, value pages are stored
-transposed, ``[pages + 1, kv_heads, head_dim, page_size]``, in the engine's type, zeroed once
-(page 0, the null page, stays zero and is never written).  Zero-init follows
-``jllm/engine/paged.py:26-38``; the layout differs: the head axis comes before the slot axis
-so that one head's keys of a page are contiguous, and values are transposed so that the
-matrix-core kernels read 8 consecutive keys of one head element as 16 aligned bytes.
+Every tensor a mixer declares in its ``PagedCacheSpec`` gets ``[pages + 1, *page_shape]`` in
+its own type (the engine's by default), zeroed once (page 0, the null page, stays zero and is
+never written).  Zero-init follows ``jllm/engine/paged.py:26-38``; the layouts are the mixers'
+own (attention: ``parts.spec.kv_cache_spec``).  Nothing here knows what the tensors hold.
 """
 from __future__ import annotations
 
@@ -40,22 +38,24 @@ def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs:
         if p.cache is not None:
             if p.cache_of is None:
                 g = group_keys.index(p.cache.group_key)
-                n, h, d = num_pages[g] + 1, p.cache.num_kv_heads, p.cache.head_dim
-                mem.k_pages = torch.zeros((n, h, page_size, d), dtype=dtype, device=device)
-                mem.v_pages = torch.zeros((n, h, d, page_size), dtype=dtype, device=device)
+                for t in p.cache.tensors:
+                    kind = dtype if t.dtype is None else _STATE_DTYPES[t.dtype]
+                    mem.pages[t.name] = torch.zeros((num_pages[g] + 1, *t.page_shape(page_size)), dtype=kind, device=device)
                 mem.group, mem.writes = g, True
             else:
                 owner = memories[p.cache_of]
-                if owner.k_pages is None:
+                if not owner.pages:
                     raise ValueError(f"run {p.run} reads the cache of run {p.cache_of}, which keeps none")
                 own, other = p.cache, plan[p.cache_of].cache
-                if (own.num_kv_heads, own.head_dim) != (other.num_kv_heads, other.head_dim):
-                    raise ValueError(f"run {p.run} cannot read run {p.cache_of}'s cache: head shapes differ")
+                if own.tensors != other.tensors:
+                    raise ValueError(f"run {p.run} cannot read run {p.cache_of}'s cache: they declare different tensors "
+                                     f"({[(t.name, t.token_shape) for t in own.tensors]} against "
+                                     f"{[(t.name, t.token_shape) for t in other.tensors]})")
                 if other.window is not None and (own.window is None or own.window > other.window):
                     raise ValueError(
                         f"run {p.run} cannot read run {p.cache_of}'s cache: it needs keys that the owner's "
                         f"window of {other.window} has already given back")
-                mem.k_pages, mem.v_pages, mem.group, mem.writes = owner.k_pages, owner.v_pages, owner.group, False
+                mem.pages, mem.group, mem.writes = owner.pages, owner.group, False
         if p.state is not None:
             # one row per slot and a spare one that belongs to no request
             mem.state = torch.zeros((max_num_seqs + 1, *p.state.shape), dtype=_STATE_DTYPES[p.state.dtype], device=device)
@@ -64,5 +64,7 @@ def allocate_memories(plan, group_keys, num_pages, page_size: int, max_num_seqs:
 
 
 def cache_bytes_per_token(plan, dtype) -> int:
-    item = torch.empty((), dtype=dtype).element_size()
-    return sum(2 * p.cache.num_kv_heads * p.cache.head_dim * item for p in plan if p.cache and p.cache_of is None)
+    def item(t):
+        return torch.empty((), dtype=dtype if t.dtype is None else _STATE_DTYPES[t.dtype]).element_size()
+
+    return sum(t.elements_per_token * item(t) for p in plan if p.cache and p.cache_of is None for t in p.cache.tensors)

@@ -4,14 +4,22 @@
 #include "common.h"
 
 // ---------------------------------------------------------------- embedding gather
-// h[t, :] = float(table[ids[t], :]).  One block per token.
+// h[t, :] = float(table[ids[t], :]).  One block per token.  An id outside [0, rows) reads nothing:
+// its row of h becomes NaN (ids may come straight from a sampling kernel on the device, which answers
+// `rows` for a row of logits without a maximum; the host reports that row when it sees the id).
 template <typename T>
 __global__ void embedding_kernel(float* __restrict__ h, const T* __restrict__ table,
-                                 const int* __restrict__ ids, int hidden) {
+                                 const int* __restrict__ ids, int hidden, int rows) {
   const long long t = blockIdx.x;
-  const T* row = table + (long long)ids[t] * hidden;
+  const int id = ids[t];
+  const bool inside = id >= 0 && id < rows;
+  const T* row = table + (long long)(inside ? id : 0) * hidden;
   float* out = h + t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) out[i] = to_f32(row[i]);
+  const float nan = __builtin_nanf("");
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = to_f32(row[i]);
+    out[i] = inside ? v : nan;
+  }
 }
 
 // ---------------------------------------------------------------- residual add + RMSNorm
@@ -355,10 +363,10 @@ __global__ void add_bias_kernel(T* __restrict__ y, const float* __restrict__ bia
 
 #define DEFINE_ELEMENTWISE(SUF, T)                                                                  \
   extern "C" int jv_embedding_##SUF(float* h, const void* table, const int* ids, int n_tokens,      \
-                                    int hidden, void* stream) {                                     \
+                                    int hidden, int rows, void* stream) {                           \
     if (n_tokens <= 0) return 0;                                                                    \
     hipLaunchKernelGGL(embedding_kernel<T>, dim3(n_tokens), dim3(256), 0, (hipStream_t)stream, h,   \
-                       (const T*)table, ids, hidden);                                               \
+                       (const T*)table, ids, hidden, rows);                                         \
     return JV_LAUNCH_CHECK();                                                                       \
   }                                                                                                 \
   extern "C" int jv_add_rmsnorm_##SUF(float* h, const void* delta, const float* w, void* out,       \

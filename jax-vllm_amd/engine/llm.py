@@ -133,7 +133,11 @@ class Engine:
             if self._ahead is not None and sampled:
                 drawn = self._ahead.launch(logits, temps, keys)
             else:
-                tokens = self._sample(logits, temps, keys)
+                try:
+                    tokens = self._sample(logits, temps, keys)
+                except Exception:
+                    self._drop(items)
+                    raise
         self._count(items)
         # the step after this one, if it is known already, goes to the GPU before this one's tokens are awaited
         following = None
@@ -144,7 +148,12 @@ class Engine:
                 temps, keys = self._draw_arguments(nxt, ahead_by=1)
                 following = _StepUnderWay(nxt, self._ahead.launch(logits, temps, keys))
         if drawn is not None:
-            tokens = self._ahead.finish(drawn)
+            try:
+                tokens = self._ahead.finish(drawn)
+            except Exception:
+                # a step started ahead has run on a token nobody can use: it is never looked at
+                self._drop(items)
+                raise
         events = []
         for item in items:
             tok = tokens[row_of[id(item)]] if item.samples else None
@@ -161,6 +170,16 @@ class Engine:
                     self._ahead.commit(item.request.request_id, item.request.output_ids[-1])
             self._under_way = following
         return events
+
+    def _drop(self, items: list) -> None:
+        """No token could be chosen for this step (a row of logits without a maximum): the cache
+        already holds the step's tokens, the requests do not, so its requests end here and give back
+        what they hold, also what a step started ahead has reserved; the others go on."""
+        for item in items:
+            req = item.request
+            if not req.finished:
+                self.scheduler.finish(req)
+            self.requests.pop(req.request_id, None)
 
     def abort_all(self) -> None:
         """Drop every waiting and running request and give back what they hold."""

@@ -69,14 +69,14 @@ def _f32(t, name: str, n: int | None = None) -> None:
 
 # --------------------------------------------------------------------------- embedding
 def embedding(h: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
-    """h[t] = float(table[ids[t]]); ids must already be checked to lie in [0, rows)."""
+    """h[t] = float(table[ids[t]]).  An id outside [0, rows) reads nothing and makes its row NaN."""
     _dev(h, table, ids)
     n, hidden = h.shape
     _f32(h, "h")
     _i32(ids, "ids", n)
     _need(table.dim() == 2 and table.shape[1] == hidden, "table width differs from h")
     fn = getattr(library.core(), f"jv_embedding_{_suffix(table.dtype)}")
-    _check(fn(_ptr(h), _ptr(table), _ptr(ids), c_int(n), c_int(hidden), _stream()), "embedding")
+    _check(fn(_ptr(h), _ptr(table), _ptr(ids), c_int(n), c_int(hidden), c_int(table.shape[0]), _stream()), "embedding")
 
 
 # --------------------------------------------------------------------------- norms

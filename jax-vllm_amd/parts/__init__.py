@@ -1,7 +1,8 @@
 from . import attention, block, embedding, mlp, norm, rotary  # noqa: F401  (register the built-in parts)
 from .model import DecoderModel, Layer, RunMemoryPlan
 from .spec import (
-    KVCacheSpec,
+    PagedCacheSpec,
+    PagedTensorSpec,
     LayerMemory,
     LayerRun,
     LayerSpec,
@@ -12,10 +13,11 @@ from .spec import (
     TensorSpec,
     build_part,
     is_replayable,
+    kv_cache_spec,
     register_part,
 )
 
 __all__ = [
-    "DecoderModel", "Layer", "RunMemoryPlan", "KVCacheSpec", "LayerMemory", "LayerRun", "LayerSpec", "ModelSpec",
+    "DecoderModel", "Layer", "RunMemoryPlan", "PagedCacheSpec", "PagedTensorSpec", "kv_cache_spec", "LayerMemory", "LayerRun", "LayerSpec", "ModelSpec",
     "PartSpec", "StateSpec", "StepContext", "TensorSpec", "build_part", "is_replayable", "register_part",
 ]

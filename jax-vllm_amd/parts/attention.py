@@ -16,8 +16,8 @@ from typing import Optional
 import torch
 
 from ..ops import kernels as K
-from .spec import (KVCacheSpec, LayerMemory, PartSpec, StepContext, TensorSpec, build_part, is_replayable,
-                   register_part)
+from .spec import (LayerMemory, PagedCacheSpec, PartSpec, StepContext, TensorSpec, build_part, is_replayable,
+                   kv_cache_spec, register_part)
 
 
 class GroupedQueryAttention:
@@ -32,6 +32,9 @@ class GroupedQueryAttention:
         self.window = int(window) if window else None
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
         self.position = build_part("position", position) if position is not None else None
+        # what the position part asks of this mixer's kernels: a rotation of q and k by position
+        # (rotary_dim, interleaved), or nothing (a part that acts elsewhere, or no part at all)
+        self.rotation = self.position.as_rotation() if self.position is not None else None
         self.qkv_bias, self.o_bias = bool(qkv_bias), bool(o_bias)
         self.w_qkv = self.w_o = self.q_norm = self.k_norm = self.b_qkv = self.b_o = None
 
@@ -61,8 +64,8 @@ class GroupedQueryAttention:
             t["o_proj.bias"] = TensorSpec((self.hidden_size,), role="vector")
         return t
 
-    def cache_spec(self) -> Optional[KVCacheSpec]:
-        return KVCacheSpec(self.nkv, self.d, self.window)
+    def cache_spec(self) -> Optional[PagedCacheSpec]:
+        return kv_cache_spec(self.nkv, self.d, self.window)
 
     def state_spec(self):
         return None
@@ -82,25 +85,25 @@ class GroupedQueryAttention:
         if self.position is not None:
             self.position.bind({}, dtype, self.w_o.device)
 
+    def _qkv_parts_ok(self) -> bool:
+        """Whether the kernel behind the qkv product (norm, rotation, page write) adds float partial
+        products itself: decided by sizes and the declared rotation alone, so the same answer holds
+        when the norm before asks and when the product runs."""
+        rotary_dim, interleaved = self.rotation if self.rotation is not None else (0, False)
+        return K.rope_takes_parts(self.dtype, self.d, interleaved, rotary_dim, self.rotation is not None)
+
     def takes_unscaled_rows(self, n_rows: int) -> bool:
         """x goes into the qkv product and nowhere else: the norm before may leave its scale to that product."""
-        if self.position is None:
-            partial_ok = K.rope_takes_parts(self.dtype, self.d, False, 0, False)
-        elif hasattr(self.position, "rotary_dim") and hasattr(self.position, "interleaved"):
-            partial_ok = K.rope_takes_parts(self.dtype, self.d, self.position.interleaved, self.position.rotary_dim, True)
-        else:
-            return False        # an encoding that tells its rotation only step by step: the product's plan is not known here
-        return K.linear_takes_unscaled_rows(n_rows, self.w_qkv, partial_ok=partial_ok, partial_max_width=None)
+        return K.linear_takes_unscaled_rows(n_rows, self.w_qkv, partial_ok=self._qkv_parts_ok(), partial_max_width=None)
 
     # ---- one step
     def forward(self, x, ctx: StepContext, mem: LayerMemory) -> torch.Tensor:
         n = x.shape[0]
-        cos_sin, rotary_dim, interleaved = (
-            self.position.fused_arguments(ctx) if self.position is not None else (None, 0, False)
-        )
+        rotary_dim, interleaved = self.rotation if self.rotation is not None else (0, False)
+        cos_sin = self.position.rotation_table(ctx) if self.rotation is not None else None
         # at few rows the projection may come as float partial products, which the next kernel adds
         qkv = K.linear(x, self.w_qkv, partial_max_width=None,       # the rotation kernel adds parts of any width
-                       partial_ok=K.rope_takes_parts(x.dtype, self.d, interleaved, rotary_dim, cos_sin is not None))
+                       partial_ok=self._qkv_parts_ok())
         if self.b_qkv is not None:
             K.add_bias(qkv, self.b_qkv)
         parts = None
@@ -110,7 +113,7 @@ class GroupedQueryAttention:
         K.qk_norm_rope_write(
             qkv, ctx.slot_mappings[mem.group] if writes else None, self.q_norm, self.k_norm,
             self.qk_norm_eps or 0.0, cos_sin, rotary_dim, interleaved,
-            mem.k_pages if writes else None, mem.v_pages if writes else None, ctx.page_size,
+            mem.pages["k"] if writes else None, mem.pages["v"] if writes else None, ctx.page_size,
             self.nq, self.nkv, self.d, parts=parts,
         )
         out = torch.empty((n, self.nq * self.d), dtype=x.dtype, device=x.device)

@@ -134,7 +134,7 @@ def run(att, out, qkv, ctx, mem) -> None:
     q_row_stride = (att.nq + 2 * att.nkv) * att.d
     if not K.mfma_attention_supported(qkv.dtype, att.d, ctx.page_size):
         K.paged_attention_generic(
-            out, qkv, q_row_stride, mem.k_pages, mem.v_pages, ctx.block_tables[mem.group], ctx.token_req,
+            out, qkv, q_row_stride, mem.pages["k"], mem.pages["v"], ctx.block_tables[mem.group], ctx.token_req,
             ctx.positions, att.nq, att.nkv, att.d, att.scale, att.window or 0,
         )
         return
@@ -144,10 +144,10 @@ def run(att, out, qkv, ctx, mem) -> None:
         plan = ctx.plans[key] = plan_mfma(ctx, att.nq, att.nkv, att.d, att.window or 0, qkv.device)
     tables = ctx.block_tables[mem.group]
     if plan.n_prefill:
-        K.attn_prefill_mfma(out, qkv, q_row_stride, mem.k_pages, mem.v_pages, tables, ctx.cu_seqlens,
+        K.attn_prefill_mfma(out, qkv, q_row_stride, mem.pages["k"], mem.pages["v"], tables, ctx.cu_seqlens,
                             ctx.context_lens, plan.prefill_work, plan.n_prefill, att.nq, att.nkv, att.d, att.scale,
                             att.window or 0)
     if plan.n_decode:
-        K.attn_decode_mfma(out, qkv, q_row_stride, mem.k_pages, mem.v_pages, tables, ctx.cu_seqlens,
+        K.attn_decode_mfma(out, qkv, q_row_stride, mem.pages["k"], mem.pages["v"], tables, ctx.cu_seqlens,
                            ctx.context_lens, plan.decode_work, plan.n_decode, att.nq, att.nkv, att.d, att.scale,
                            att.window or 0, plan.num_splits, plan.scratch)

@@ -36,17 +36,22 @@ class PreNormBlock:
             part.bind({k[len(name) + 1:]: v for k, v in tensors.items() if k.startswith(name + ".")}, dtype)
 
     def forward(self, h, delta, mixer, feed_forward, ctx, mem):
-        # a part that says so (``takes_unscaled_rows(rows)``) may get ``K.UnscaledRows`` from the norm
         n = h.shape[0]
-        x = self.mixer_norm.add_norm(h, delta, unscaled_ok=_takes_unscaled(mixer, n))
+        x = _add_norm(self.mixer_norm, h, delta, mixer, n)
         a = mixer.forward(x, ctx, mem)
-        y = self.feed_forward_norm.add_norm(h, a, unscaled_ok=_takes_unscaled(feed_forward, n))
+        y = _add_norm(self.feed_forward_norm, h, a, feed_forward, n)
         return feed_forward.forward(y, ctx)
 
 
-def _takes_unscaled(part, n_rows: int) -> bool:
-    ask = getattr(part, "takes_unscaled_rows", None)
-    return bool(ask is not None and ask(n_rows))
+def _add_norm(norm, h, delta, reader, n_rows: int):
+    """``norm.add_norm(h, delta)``.  Only where both sides have said so, the norm may hand on
+    ``K.UnscaledRows``: a norm part declares ``may_leave_scale = True`` (its ``add_norm`` takes
+    ``unscaled_ok``), a reader part answers ``takes_unscaled_rows(rows)``.  Parts that declare
+    neither see the plain interface."""
+    ask = getattr(reader, "takes_unscaled_rows", None)
+    if getattr(norm, "may_leave_scale", False) and ask is not None and ask(n_rows):
+        return norm.add_norm(h, delta, unscaled_ok=True)
+    return norm.add_norm(h, delta)
 
 
 register_part("block", "prenorm", PreNormBlock)

@@ -22,8 +22,10 @@ class TokenEmbedding:
     def bind(self, tensors: dict, dtype: torch.dtype) -> None:
         self.weight = tensors["weight"]
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
-        """Float residual stream [tokens, hidden] of the rows ``ids`` (int32, already range-checked)."""
+    def forward(self, ids: torch.Tensor, ctx=None) -> torch.Tensor:
+        """Float residual stream [tokens, hidden] of the rows ``ids`` (int32; an id outside the table
+        gives a row of NaN).  ``ctx`` is the step's ``StepContext`` (positions, token -> request, ...);
+        this embedding needs none of it."""
         h = torch.empty((ids.numel(), self.hidden_size), dtype=torch.float32, device=ids.device)
         K.embedding(h, self.weight, ids)
         return h

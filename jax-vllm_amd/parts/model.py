@@ -12,7 +12,7 @@ from typing import Optional
 
 import torch
 
-from .spec import (KVCacheSpec, LayerMemory, LayerSpec, ModelSpec, StateSpec, StepContext, TensorSpec, build_part,
+from .spec import (PagedCacheSpec, LayerMemory, LayerSpec, ModelSpec, StateSpec, StepContext, TensorSpec, build_part,
                    is_replayable)
 
 
@@ -53,7 +53,7 @@ class RunMemoryPlan:
 
     run: int
     layer: int
-    cache: Optional[KVCacheSpec]
+    cache: Optional[PagedCacheSpec]
     state: Optional[StateSpec]
     cache_of: Optional[int]
 
@@ -121,7 +121,7 @@ class DecoderModel:
     def forward(self, token_ids: torch.Tensor, ctx: StepContext, memories: list, logit_rows: torch.Tensor):
         """Runs the step's tokens through every schedule entry; returns float logits
         [len(logit_rows), vocab] for the token rows named by ``logit_rows`` (int32)."""
-        h = self.embedding.forward(token_ids)
+        h = self.embedding.forward(token_ids, ctx)
         delta = None
         for run, mem in zip(self.spec.schedule, memories):
             layer = self.layers[run.layer]

@@ -15,6 +15,7 @@ from .spec import TensorSpec, register_part
 
 class RMSNorm:
     replayable = True
+    may_leave_scale = True     # ``add_norm`` takes ``unscaled_ok`` (a norm part without this attribute is never asked)
 
     def __init__(self, size: int, eps: float):
         self.size, self.eps = int(size), float(eps)

@@ -39,14 +39,19 @@ class RotaryEncoding:
     def bind(self, tensors: dict, dtype: torch.dtype, device=None) -> None:
         self.inv_freq = self.inverse_frequencies().to(device or "cuda").contiguous()
 
-    def fused_arguments(self, ctx):
-        """(cos/sin table of the step's positions, rotary_dim, interleaved) for the
-        attention-input kernel."""
+    def as_rotation(self):
+        """(rotary_dim, interleaved): this encoding is a rotation of q and k by position, which the
+        mixer's own kernel applies from ``rotation_table``.  A position part that asks nothing of
+        the mixer's kernels answers None."""
+        return self.rotary_dim, self.interleaved
+
+    def rotation_table(self, ctx):
+        """Float cos/sin table of the step's positions for the attention-input kernel."""
         key = ("rope_table", self.theta, self.rotary_dim)
         table = ctx.extras.get(key)
         if table is None:
             table = ctx.extras[key] = K.rope_table(ctx.positions, self.inv_freq)
-        return table, self.rotary_dim, self.interleaved
+        return table
 
 
 register_part("position", "rotary", RotaryEncoding)

@@ -37,17 +37,66 @@ class TensorSpec:
 
 
 @dataclass(frozen=True)
-class KVCacheSpec:
-    """Keys and values in pages.  ``window`` None: every earlier key is read ("full");
-    otherwise only the last ``window`` keys are, and older pages are given back."""
+class PagedTensorSpec:
+    """One tensor that a mixer keeps per cached token, in pages.
 
-    num_kv_heads: int
-    head_dim: int
+    ``token_shape`` is what one token stores (e.g. ``(kv_heads, head_dim)``).  A page holds
+    ``page_size`` tokens; ``slot_axis`` says where the axis of the tokens of a page is put among
+    the token's own axes: 0 gives pages ``[page_size, *token_shape]``, ``len(token_shape)`` puts
+    it last (a page's tokens are then contiguous per element).  The storage is
+    ``[pages + 1, *page_shape]`` with page 0 the null page.  ``dtype`` None: the engine's compute
+    type; otherwise "float32", "bfloat16" or "int32".
+    """
+
+    name: str
+    token_shape: tuple
+    slot_axis: int = 0
+    dtype: Optional[str] = None
+
+    def __post_init__(self):
+        if not 0 <= self.slot_axis <= len(self.token_shape):
+            raise ValueError(f"cache tensor {self.name!r}: slot axis {self.slot_axis} outside 0..{len(self.token_shape)}")
+
+    def page_shape(self, page_size: int) -> tuple:
+        shape = list(self.token_shape)
+        shape.insert(self.slot_axis, int(page_size))
+        return tuple(shape)
+
+    @property
+    def elements_per_token(self) -> int:
+        n = 1
+        for s in self.token_shape:
+            n *= int(s)
+        return n
+
+
+@dataclass(frozen=True)
+class PagedCacheSpec:
+    """What a mixer keeps per token in pages: the tensors it declares (a page of each for every
+    page id) and which earlier tokens it reads.  ``window`` None: every earlier token is read
+    ("full"); otherwise only the last ``window`` are, and older pages are given back.  Mixers with
+    the same need share a page pool and a block table (a *group*), whatever tensors they keep."""
+
+    tensors: tuple
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [t.name for t in self.tensors]
+        if len(set(names)) != len(names) or not names:
+            raise ValueError(f"a paged cache needs tensors with distinct names, got {names}")
 
     @property
     def group_key(self) -> tuple:
         return ("window", self.window) if self.window else ("full",)
+
+
+def kv_cache_spec(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> PagedCacheSpec:
+    """Keys and values of grouped-query attention in the layout its kernels read: a key page is
+    ``[kv_heads, page_size, head_dim]`` (one head's keys of a page are contiguous), a value page
+    is transposed, ``[kv_heads, head_dim, page_size]`` (8 consecutive keys of one head element are
+    16 aligned bytes)."""
+    shape = (int(num_kv_heads), int(head_dim))
+    return PagedCacheSpec((PagedTensorSpec("k", shape, slot_axis=1), PagedTensorSpec("v", shape, slot_axis=2)), window)
 
 
 @dataclass(frozen=True)
@@ -62,15 +111,14 @@ class StateSpec:
 class LayerMemory:
     """What the cache manager hands one layer run.
 
-    k_pages [pages, kv_heads, page_size, head_dim], v_pages [pages, kv_heads, head_dim,
-    page_size] (transposed), or None; ``group`` says which
-    block table / slot mapping of the step applies; ``writes`` is False for a run that reads
-    another run's cache.  ``state`` is [slots + 1, *shape] or None; its last row belongs to no
-    request (rows that pad a captured step point there).
+    ``pages``: the storage of every tensor the run's mixer declared in its ``PagedCacheSpec``, by
+    name, each ``[pages + 1, *page_shape]`` (empty for a mixer without a paged cache);
+    ``group`` says which block table / slot mapping of the step applies; ``writes`` is False for
+    a run that reads another run's cache.  ``state`` is [slots + 1, *shape] or None; its last row
+    belongs to no request (rows that pad a captured step point there).
     """
 
-    k_pages: Optional[torch.Tensor] = None
-    v_pages: Optional[torch.Tensor] = None
+    pages: dict = field(default_factory=dict)
     group: int = 0
     writes: bool = True
     state: Optional[torch.Tensor] = None

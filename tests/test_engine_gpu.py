@@ -581,7 +581,7 @@ def test_attention_part_alone(folders, dtype, biased):
     block gives the reference with the bias as a last column of its weight."""
     from jax_vllm_amd.cache import CacheManager
     from jax_vllm_amd.cache.storage import allocate_memories
-    from jax_vllm_amd.parts import KVCacheSpec, PartSpec, build_part
+    from jax_vllm_amd.parts import PartSpec, build_part, kv_cache_spec
     from jax_vllm_amd.parts.model import RunMemoryPlan
     from jax_vllm_amd.parts.spec import StepContext
 
@@ -598,7 +598,8 @@ def test_attention_part_alone(folders, dtype, biased):
     ws = {n: v.to(tdt).float() for n, v in ws.items()}
     att.bind({n: v.to(tdt if att.tensors()[n].role == "matrix" else torch.float32).cuda() for n, v in ws.items()}, tdt)
     plan = [RunMemoryPlan(0, 0, att.cache_spec(), None, None)]
-    assert att.cache_spec() == KVCacheSpec(nkv, d, None)
+    assert att.cache_spec() == kv_cache_spec(nkv, d, None)
+    assert [(t.name, t.page_shape(ps)) for t in att.cache_spec().tensors] == [("k", (nkv, ps, d)), ("v", (nkv, d, ps))]
     mem = allocate_memories(plan, [("full",)], 16, ps, 2, tdt, "cuda")[0]
     cache = CacheManager([("full",)], ps, 16, 2, enable_prefix_cache=False)
     cfg = dict(num_heads=nq, num_kv_heads=nkv, head_dim=d, rms_norm_eps=1e-5, rope_theta=1e4)
@@ -949,13 +950,16 @@ class LinearFrequencyRotation:
     def bind(self, tensors, dtype, device=None):
         self.freq = (torch.arange(1, self.rotary_dim // 2 + 1, dtype=torch.float32) * self.step).to(device or "cuda")
 
-    def fused_arguments(self, ctx):
+    def as_rotation(self):
+        return self.rotary_dim, True
+
+    def rotation_table(self, ctx):
         from jax_vllm_amd.ops import kernels as K
 
         key = ("linear_frequency_table", self.rotary_dim, self.step)
         if key not in ctx.extras:
             ctx.extras[key] = K.rope_table(ctx.positions, self.freq)
-        return ctx.extras[key], self.rotary_dim, True
+        return ctx.extras[key]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -1057,3 +1061,221 @@ def test_toy_routed_feed_forward_and_toy_position_encoding(dtype):
         at += n
     assert at == len(toks)
     check_logits(dtype, np.concatenate(got), want)
+
+
+# ------------------------------------------------------------------ an embedding that reads the step's positions; a mixer with a cache of its own shape
+class PositionedEmbedding:
+    """A toy embedding, defined and registered here: token row plus a learned row per absolute
+    position.  It takes the positions from the step's context on the device, so it may be replayed."""
+
+    replayable = True
+
+    def __init__(self, vocab_size: int, hidden_size: int, max_positions: int):
+        self.v, self.h, self.n = vocab_size, hidden_size, max_positions
+
+    def tensors(self):
+        from jax_vllm_amd.parts import TensorSpec
+
+        return {"weight": TensorSpec((self.v, self.h)), "positions.weight": TensorSpec((self.n, self.h))}
+
+    def bind(self, tensors, dtype):
+        self.weight, self.rows = tensors["weight"], tensors["positions.weight"]
+
+    def forward(self, ids, ctx):
+        return self.weight[ids.long()].float() + self.rows[ctx.positions.long()].float()
+
+
+class LatentMeanMixer:
+    """A toy mixer with a paged cache that is no key/value pair: per token it stores ONE latent
+    vector of ``latent`` floats (always float32, token-major pages), and its output at a token is a
+    projection of the mean of the latents of all tokens up to it, read back from the pages through
+    the block table.  Plans on the host; never replayed."""
+
+    def __init__(self, hidden_size: int, latent: int):
+        self.h, self.r = hidden_size, latent
+
+    def tensors(self):
+        from jax_vllm_amd.parts import TensorSpec
+
+        return {"down.weight": TensorSpec((self.r, self.h)), "up.weight": TensorSpec((self.h, self.r))}
+
+    def cache_spec(self):
+        from jax_vllm_amd.parts import PagedCacheSpec, PagedTensorSpec
+
+        return PagedCacheSpec((PagedTensorSpec("latent", (self.r,), slot_axis=0, dtype="float32"),))
+
+    def state_spec(self):
+        return None
+
+    def bind(self, tensors, dtype):
+        self.down, self.up = tensors["down.weight"], tensors["up.weight"]
+
+    def forward(self, x, ctx, mem):
+        store = mem.pages["latent"]                       # [pages + 1, page_size, latent]
+        flat = store.view(-1, self.r)
+        if mem.writes:                                    # a run that reads another run's cache stores nothing
+            flat[ctx.slot_mappings[mem.group].long()] = (x @ self.down.t()).float()
+        out = torch.empty_like(x)
+        tables = ctx.block_tables[mem.group]
+        at = 0
+        for i, (q, c) in enumerate(zip(ctx.q_lens_host, ctx.context_lens_host)):
+            seen = store[tables[i].long()].reshape(-1, self.r)[:c + q]        # the request's latents in order
+            means = torch.cumsum(seen, 0)[c:] / torch.arange(c + 1, c + q + 1, device=x.device)[:, None]
+            out[at:at + q] = (means.to(x.dtype) @ self.up.t()).to(x.dtype)
+            at += q
+        return out
+
+
+def _bound_toy(name, spec_builder, dtype, seed, scale=0.2):
+    from jax_vllm_amd.config import register_architecture, resolve
+    from jax_vllm_amd.parts import DecoderModel
+    from jax_vllm_amd.weights.loader import TORCH_DTYPES, target_dtype
+
+    register_architecture(name, lambda c: c, spec_builder)
+    arch, cfg, _ = resolve({"architectures": [name]})
+    model = DecoderModel(arch.build_spec(cfg))
+    g = torch.Generator().manual_seed(seed)
+    compute = TORCH_DTYPES[dtype]
+    w = {n: ((scale * torch.randn(ts.shape, generator=g)) if ts.role == "matrix" else 1 + 0.1 * torch.randn(ts.shape, generator=g))
+         .to(torch.bfloat16).float() for n, ts in model.tensor_specs().items()}
+    model.bind({n: v.cuda().to(target_dtype(model.tensor_specs()[n].role, compute)) for n, v in w.items()}, compute)
+    return model, w
+
+
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs-on"])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_embedding_with_learned_positions_and_attention_without_rotation(dtype, graphs):
+    """The embedding part gets the step's context: a learned row per absolute position is added
+    there, and the attention runs with no position part at all.  Nothing of the package changes."""
+    from jax_vllm_amd.parts import LayerRun, LayerSpec, ModelSpec, PartSpec, register_part
+
+    register_part("embedding", "positioned_embedding", PositionedEmbedding)
+    hidden, vocab, inter, heads, kvh, d, eps, npos = 56, 75, 72, 4, 2, 16, 1e-5, 128
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": eps})
+    att = PartSpec("gqa_attention", dict(hidden_size=hidden, num_heads=heads, num_kv_heads=kvh, head_dim=d, qk_norm_eps=eps))
+
+    def build(_cfg):
+        return ModelSpec(
+            vocab_size=vocab, hidden_size=hidden,
+            embedding=PartSpec("positioned_embedding", {"vocab_size": vocab, "hidden_size": hidden, "max_positions": npos}),
+            embedding_prefix="emb.", final_norm=norm, final_norm_prefix="norm.",
+            head=PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": hidden}), head_prefix="head.",
+            layers=[LayerSpec(f"l{i}.", att, PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter}),
+                              PartSpec("prenorm", {"norm": norm}), "att.", "ff.") for i in range(2)],
+            schedule=[LayerRun(0), LayerRun(1)])
+
+    model, w = _bound_toy("ToyPositionedModel", build, dtype, 31)
+    assert model.replayable()
+
+    def plain(tokens):
+        t = len(tokens)
+        h = w["emb.weight"][torch.tensor(tokens)] + w["emb.positions.weight"][:t]
+        for i in (0, 1):
+            p = f"l{i}.att"
+            x = P.rms_norm(w[f"l{i}.input_layernorm.weight"], eps, h)
+            q = P.rms_norm(w[f"{p}.q_norm.weight"], eps, (x @ w[f"{p}.q_proj.weight"].T).reshape(t, heads, d).transpose(0, 1))
+            k = P.rms_norm(w[f"{p}.k_norm.weight"], eps, (x @ w[f"{p}.k_proj.weight"].T).reshape(t, kvh, d).transpose(0, 1))
+            v = (x @ w[f"{p}.v_proj.weight"].T).reshape(t, kvh, d).transpose(0, 1)
+            o = P.attention_core(q, k, v, P.causal_mask(t, t)).transpose(0, 1).reshape(t, heads * d)
+            h = h + o @ w[f"{p}.o_proj.weight"].T
+            m = P.rms_norm(w[f"l{i}.post_attention_layernorm.weight"], eps, h)
+            h = h + P.swiglu(w[f"l{i}.ff.gate_proj.weight"], w[f"l{i}.ff.up_proj.weight"], w[f"l{i}.ff.down_proj.weight"], m)
+        return (P.rms_norm(w["norm.weight"], eps, h) @ w["head.weight"].T).numpy()
+
+    core = make_core(None, dtype, 8, pages=30, seqs=3, model=model, graphs=graphs)
+    rng = np.random.default_rng(9)
+    reqs = {r: rng.integers(0, vocab, size=n).tolist() for r, n in (("a", 60), ("b", 41))}
+    # without its position rows the model would not tell a sequence from a permutation of it: the
+    # oracle's answer must depend on them
+    assert np.abs(plain(reqs["b"])[-1] - plain(reqs["b"][::-1][:-1] + reqs["b"][-1:])[-1]).max() > 1e-3
+    fed, got = {r: 0 for r in reqs}, {r: [] for r in reqs}
+    for r in reqs:
+        core.start_request(r)
+    cuts = [[("a", 9)], [("a", 30), ("b", 22)], [("a", 1), ("b", 2)]] + [[("a", 1), ("b", 1)]] * 17 + [[("a", 1)]] * 3
+    for step in cuts:
+        out = core.run([entry(r, reqs[r][fed[r]:fed[r] + n]) for r, n in step]).cpu().numpy()
+        at = 0
+        for r, n in step:
+            got[r].append(out[at:at + n])
+            at, fed[r] = at + n, fed[r] + n
+    assert (core.graph_replays > 10) == graphs
+    for r in reqs:
+        assert fed[r] == len(reqs[r])
+        check_logits(dtype, np.concatenate(got[r]), plain(reqs[r]), what=r)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_declares_a_paged_cache_of_its_own_shape(dtype):
+    """A mixer says what it keeps per token; the storage gives it exactly that (one float32 tensor,
+    token-major pages), in a page group that it shares with an attention layer (same need: all
+    earlier tokens), and pages are taken again after requests end."""
+    from jax_vllm_amd.parts import LayerRun, LayerSpec, ModelSpec, PartSpec, register_part
+
+    register_part("mixer", "latent_mean", LatentMeanMixer)
+    hidden, vocab, inter, latent, eps, ps = 48, 66, 64, 12, 1e-5, 8
+    norm = PartSpec("rmsnorm", {"size": hidden, "eps": eps})
+    att = PartSpec("gqa_attention", dict(hidden_size=hidden, num_heads=3, num_kv_heads=1, head_dim=16, qk_norm_eps=eps,
+                                         position=PartSpec("rotary", {"head_dim": 16, "theta": 1e4})))
+    toy = PartSpec("latent_mean", {"hidden_size": hidden, "latent": latent})
+    ffn = PartSpec("gated_mlp", {"hidden_size": hidden, "intermediate_size": inter})
+
+    def build(_cfg):
+        return ModelSpec(
+            vocab_size=vocab, hidden_size=hidden,
+            embedding=PartSpec("token_embedding", {"vocab_size": vocab, "hidden_size": hidden}), embedding_prefix="emb.",
+            final_norm=norm, final_norm_prefix="norm.", head=PartSpec("linear_head", {"vocab_size": vocab, "hidden_size": hidden}),
+            head_prefix="head.", tie_head_to_embedding=True,
+            layers=[LayerSpec(f"l{i}.", mixer, ffn, PartSpec("prenorm", {"norm": norm}), "mix.", "ffn.")
+                    for i, mixer in enumerate([toy, att])],
+            schedule=[LayerRun(0), LayerRun(1), LayerRun(0, cache_of=0)])    # the third run reads the first run's latents
+
+    model, w = _bound_toy("ToyLatentModel", build, dtype, 37)
+    core = make_core(None, dtype, ps, pages=12, seqs=3, model=model)
+    assert core.group_keys == [("full",)]
+    toy_mem, att_mem, reader = core.memories
+    assert list(toy_mem.pages) == ["latent"] and toy_mem.pages["latent"].shape == (13, ps, latent)
+    assert toy_mem.pages["latent"].dtype == torch.float32
+    assert sorted(att_mem.pages) == ["k", "v"] and att_mem.pages["k"].dtype == core.dtype
+    assert reader.pages is toy_mem.pages and not reader.writes
+    item = 4 if dtype == "float32" else 2
+    assert core.kv_bytes_per_token == latent * 4 + 2 * 16 * item
+
+    def plain(tokens):
+        t = len(tokens)
+        c = dict(num_heads=3, num_kv_heads=1, head_dim=16, rms_norm_eps=eps, rope_theta=1e4)
+        h = w["emb.weight"][torch.tensor(tokens)]
+        first = None
+        for run, i in enumerate((0, 1, 0)):
+            x = P.rms_norm(w[f"l{i}.input_layernorm.weight"], eps, h)
+            if i == 1:
+                a = P.attention_block(w, "l1.mix", c, x, torch.arange(t))
+            else:
+                lat = x @ w["l0.mix.down.weight"].T
+                first = lat if first is None else first          # the reader run mixes the owner's latents
+                a = (torch.cumsum(first, 0) / torch.arange(1, t + 1)[:, None]) @ w["l0.mix.up.weight"].T
+            h = h + a
+            m = P.rms_norm(w[f"l{i}.post_attention_layernorm.weight"], eps, h)
+            h = h + P.swiglu(w[f"l{i}.ffn.gate_proj.weight"], w[f"l{i}.ffn.up_proj.weight"], w[f"l{i}.ffn.down_proj.weight"], m)
+        return (P.rms_norm(w["norm.weight"], eps, h) @ w["emb.weight"].T).numpy()
+
+    rng = np.random.default_rng(10)
+    reqs = {r: rng.integers(0, vocab, size=n).tolist() for r, n in (("a", 37), ("b", 30), ("c", 44), ("d", 25))}
+    fed, got = {r: 0 for r in reqs}, {r: [] for r in reqs}
+    cuts = [[("a", 11)], [("a", 2), ("b", 17)], [("a", 24), ("b", 1)], [("b", 12)],       # a and b end: 9 of 12 pages go back
+            [("c", 30)], [("c", 1), ("d", 9)], [("c", 13), ("d", 16)]]
+    for step in cuts:
+        for r, _ in step:
+            if not core.has_request(r):
+                core.start_request(r)
+        out = core.run([entry(r, reqs[r][fed[r]:fed[r] + n]) for r, n in step]).cpu().numpy()
+        at = 0
+        for r, n in step:
+            got[r].append(out[at:at + n])
+            at, fed[r] = at + n, fed[r] + n
+            if fed[r] == len(reqs[r]):
+                core.finish_request(r)
+        core.cache.check_invariants()
+    assert core.cache.num_free_pages(0) == 12
+    for r in reqs:
+        assert fed[r] == len(reqs[r])
+        check_logits(dtype, np.concatenate(got[r]), plain(reqs[r]), what=r)

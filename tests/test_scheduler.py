@@ -465,3 +465,37 @@ def test_abort_with_a_step_under_way():
     assert eng._under_way is None and not eng.has_work()
     assert core.cache.num_free_pages() == eng.config.usable_pages
     assert eng.generate([[5, 6]], SamplingParams(max_new_tokens=5)) == [expected([5, 6], 5)]
+
+
+@pytest.mark.parametrize("with_ahead", [False, True])
+def test_a_step_whose_tokens_cannot_be_chosen_ends_its_requests_and_nothing_else(with_ahead):
+    """The sampler raises for a row of logits without a maximum.  By then the cache holds the
+    step's tokens and a step started ahead may hold a page more: the loop ends the requests of that
+    step (everything they hold goes back), raises, and serves later requests as if nothing had
+    happened."""
+    kw = dict(block_size=4, max_num_seqs=2, max_model_len=64, max_num_batched_tokens=32)
+    eng, core, ahead = make_ahead(**kw) if with_ahead else (*make(**kw), None)
+    fail_at = {"calls": 0}
+
+    def failing(fn):
+        def wrapped(arg, *more):
+            fail_at["calls"] += 1
+            if fail_at["calls"] == 4:
+                raise FloatingPointError("logits row(s) [0] of 1 hold no finite maximum")
+            return fn(arg, *more)
+        return wrapped
+
+    if with_ahead:
+        ahead.finish = failing(ahead.finish)
+    else:
+        eng._sample = failing(eng._sample)
+    a = eng.add_request([1, 2, 3], SamplingParams(max_new_tokens=10))
+    got = []
+    with pytest.raises(FloatingPointError):
+        for _ in range(10):
+            got += [e.token for e in eng.step()]
+    assert got == expected([1, 2, 3], 3)
+    assert a not in eng.requests and not eng.has_work() and eng._under_way is None
+    core.cache.check_invariants()
+    assert core.cache.num_free_pages() == eng.config.usable_pages and not core.cache.requests
+    assert eng.generate([[5, 6]], SamplingParams(max_new_tokens=5)) == [expected([5, 6], 5)]
