@@ -2,8 +2,9 @@
 
 No cache, no batching, no kernels, one function per part, nothing imported from
 the product package.  Every function follows the reference's formula and cites
-it (paths relative to the reference checkout).  Runs on CPU in float32 (or
-float64 for a tighter oracle).
+it (paths relative to the reference checkout).  Runs in float32 (or float64 for a
+tighter oracle) on the device the weights live on: the CPU, or, for the sizes of real
+models, the GPU with torch's plain float32 products (``use_exact_float32_products``).
 """
 from __future__ import annotations
 
@@ -44,6 +45,14 @@ def read_weights(folder, dtype=torch.float32) -> dict:
     return out
 
 
+def use_exact_float32_products() -> None:
+    """Forbid torch's reduced-precision modes for float32 matrix products on the GPU, so that
+    the oracle there is the same arithmetic as on the CPU (up to summation order)."""
+    torch.backends.cuda.matmul.allow_tf32 = False
+    torch.backends.cudnn.allow_tf32 = False
+    torch.set_float32_matmul_precision("highest")
+
+
 # --------------------------------------------------------------------------- parts
 def embed(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     """Row gather, no scaling: jllm/model/common.py:35-36."""
@@ -65,7 +74,7 @@ def rope_cos_sin(dim: int, theta: float, positions: torch.Tensor, dtype):
     """inv_freq[i] = theta^(-2i/dim); angles = pos * inv_freq; the half-table is
     repeated twice along the last axis: jllm/model/common.py:51-55."""
     inv_freq = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))
-    freqs = positions.to(torch.float32)[..., None] * inv_freq
+    freqs = positions.to(torch.float32)[..., None] * inv_freq.to(positions.device)
     emb = torch.cat([freqs, freqs], dim=-1)
     return torch.cos(emb).to(dtype), torch.sin(emb).to(dtype)
 
@@ -87,11 +96,11 @@ def swiglu(w_gate, w_up, w_down, x):
     return linear(w_down, torch.nn.functional.silu(linear(w_gate, x)) * linear(w_up, x))
 
 
-def causal_mask(t_q: int, t_k: int) -> torch.Tensor:
+def causal_mask(t_q: int, t_k: int, device=None) -> torch.Tensor:
     """Key j is visible to query i iff j <= (t_k - t_q) + i: jllm/model/common.py:203-214
     (with every row valid); for t_q == t_k this is the tril of common.py:163."""
-    q_idx = torch.arange(t_q)[:, None]
-    k_idx = torch.arange(t_k)[None, :]
+    q_idx = torch.arange(t_q, device=device)[:, None]
+    k_idx = torch.arange(t_k, device=device)[None, :]
     return k_idx <= (t_k - t_q) + q_idx
 
 
@@ -101,12 +110,12 @@ def attention_core(q, k, v, mask):
     jllm/model/common.py:173-178 and :191-200.  q [nq,Tq,D], k,v [nkv,Tk,D]."""
     nq, nkv, d = q.shape[0], k.shape[0], q.shape[-1]
     rep = nq // nkv
-    k = torch.repeat_interleave(k, rep, dim=0)
-    v = torch.repeat_interleave(v, rep, dim=0)
-    scores = torch.einsum("hqd,hkd->hqk", q, k) * (1.0 / math.sqrt(d))
-    scores = torch.where(mask[None], scores, torch.full_like(scores, float("-inf")))
-    probs = torch.softmax(scores, dim=-1)
-    return torch.einsum("hqk,hkd->hqd", probs, v)
+    out = []
+    for h in range(nq):      # head by head: the scores of a long sequence are [T, T] floats per head
+        scores = (q[h] @ k[h // rep].T) * (1.0 / math.sqrt(d))
+        scores = torch.where(mask, scores, torch.full_like(scores, float("-inf")))
+        out.append(torch.softmax(scores, dim=-1) @ v[h // rep])
+    return torch.stack(out)
 
 
 def attention_block(w: dict, p: str, cfg: dict, x: torch.Tensor, positions: torch.Tensor, window=None,
@@ -129,9 +138,9 @@ def attention_block(w: dict, p: str, cfg: dict, x: torch.Tensor, positions: torc
         k = apply_rope(k, cos, sin)
     else:
         k, v = shared_kv
-    mask = causal_mask(t, t)
+    mask = causal_mask(t, t, x.device)
     if window:
-        idx = torch.arange(t)
+        idx = torch.arange(t, device=x.device)
         mask = mask & (idx[None, :] > idx[:, None] - window)
     out = attention_core(q, k, v, mask)
     out = out.transpose(0, 1).reshape(t, nq * d)
@@ -154,15 +163,19 @@ def decoder_layer(w: dict, i: int, cfg: dict, h: torch.Tensor, positions: torch.
     return h
 
 
-def forward(w: dict, cfg: dict, token_ids, first_position: int = 0) -> torch.Tensor:
-    """Whole-sequence forward of one request, logits at every position [T, V]:
-    jllm/model/common.py:150-170.  lm_head is the embedding table when tied
-    (jllm/model/weights.py:143-146)."""
-    ids = torch.as_tensor(token_ids, dtype=torch.long)
-    positions = torch.arange(ids.shape[0]) + first_position
+def forward(w: dict, cfg: dict, token_ids, first_position: int = 0, rows=None) -> torch.Tensor:
+    """Whole-sequence forward of one request, logits at every position [T, V] (or only at the
+    positions ``rows``, as the reference's engine applies the head to the wanted rows only,
+    jllm/engine/generate.py:140-142): jllm/model/common.py:150-170.  lm_head is the embedding
+    table when tied (jllm/model/weights.py:143-146).  Runs where the weights are."""
+    device = w["model.embed_tokens.weight"].device
+    ids = torch.as_tensor(token_ids, dtype=torch.long, device=device)
+    positions = torch.arange(ids.shape[0], device=device) + first_position
     h = embed(w["model.embed_tokens.weight"], ids)
     for i in range(cfg["num_hidden_layers"]):
         h = decoder_layer(w, i, cfg, h, positions)
+    if rows is not None:
+        h = h[torch.as_tensor(rows, dtype=torch.long, device=device)]
     h = rms_norm(w["model.norm.weight"], cfg["rms_norm_eps"], h)
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return linear(head, h)

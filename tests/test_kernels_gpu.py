@@ -691,6 +691,56 @@ def test_attention_edges_of_visibility(edge, kernel):
                                    msg=lambda m: f"context {ctx}, query {qi}, key {key}: {m}")
 
 
+@pytest.mark.parametrize("kernel", ["prefill", "decode1", "decode4", "decode16"])
+@pytest.mark.parametrize("ctx", [8191, 16400, 32767])
+def test_mfma_attention_over_long_contexts_at_head_size_128(kernel, ctx):
+    """Heads of 128, 4 per kv head, pages of 16, behind 8 k to 32 k keys.  Among thousands of random
+    keys a missing page would change nothing that a tolerance sees, so every checked query has TWO
+    loud keys far apart (the first key, a page's last slot in the middle, a page's first slot, the
+    newest key): its output is the mean of their two values, and a key that is lost, read from a
+    wrong page or merged with a wrong weight shows as an error of half a value."""
+    nq, nkv, d, page_size = 8, 2, 128, 16
+    scale = 1.0 / math.sqrt(d)
+    bf = torch.bfloat16
+    decode = kernel.startswith("decode")
+    ql = 1 if decode else 130
+    mid = (ctx // 2) // page_size * page_size
+    pairs = [(0, ctx + ql - 1), (mid - 1, mid), (15, ctx - 16), (mid + 16, ctx // 4 * 3 + 5)]
+    g = torch.Generator().manual_seed(ctx)
+    reqs, qs, ks, vs, checked = [], [], [], [], []
+    for r, (a, b) in enumerate(pairs if decode else pairs[:2]):
+        k = torch.randn(ctx + ql, nkv, d, generator=g) * 0.1
+        v = torch.randn(ctx + ql, nkv, d, generator=g)
+        q = torch.randn(ql, nq, d, generator=g) * 0.1
+        for qi, comp in ((0, 0),) if decode else ((0, 0), (64, 1), (129, 2)):
+            hi = min(b, ctx + qi)                      # a query cannot see beyond itself
+            q[qi, :, comp] = 40.0
+            k[a, :, comp] = 40.0
+            k[hi, :, comp] = 40.0
+            checked.append((r, qi))
+        reqs.append((ctx, ql))
+        qs.append(q.to(bf).float()), ks.append(k.to(bf).float()), vs.append(v.to(bf).float())
+    k_pages, v_pages, tables = build_paged(ks, vs, page_size, seed=ctx)
+    n = len(reqs) * ql
+    out = torch.full((n, nq * d), float("nan"), dtype=bf).cuda()
+    qbuf = torch.cat([q.reshape(ql, nq * d) for q in qs]).to(bf).cuda()
+    cu = torch.tensor([i * ql for i in range(len(reqs) + 1)], dtype=torch.int32).cuda()
+    cl = torch.tensor([ctx] * len(reqs), dtype=torch.int32).cuda()
+    args = (out, qbuf, nq * d, k_pages.to(bf).cuda(), v_pages.to(bf).cuda(), tables.cuda(), cu, cl)
+    if decode:
+        splits = int(kernel[6:])
+        scratch = torch.full((max(1, K().attn_decode_scratch_floats(len(reqs), nq, splits, d)),), float("nan")).cuda()
+        K().attn_decode_mfma(*args, None, len(reqs), nq, nkv, d, scale, 0, splits, scratch)
+    else:
+        work, n_work = _prefill_work(reqs, nq // nkv, d, None, "planner")
+        K().attn_prefill_mfma(*args, work, n_work, nq, nkv, d, scale, 0)
+    got = out.double().cpu().reshape(len(reqs), ql, nq * d)
+    for r, qi in checked:
+        ref = attention_reference(qs[r][qi:qi + 1], ks[r], vs[r], torch.tensor([ctx + qi]), scale).reshape(nq * d)
+        assert float(ref.abs().max()) > 0.5            # the oracle's answer is a mean of two values, not of thousands
+        torch.testing.assert_close(got[r, qi], ref, rtol=2e-2, atol=2e-2, msg=lambda m: f"request {r}, query {qi}: {m}")
+
+
 def test_mfma_attention_ignores_garbage_past_the_context():
     """Slots of the last page beyond the context hold NaN and infinity: they must not leak."""
     nq, nkv, d, page_size = 4, 2, 64, 16

@@ -8,7 +8,7 @@ import torch
 import torch.nn.functional as F
 
 from tests.plain import qwen3_plain as P
-from tests.tiny import TINY_A, TINY_B, make_weights_dict
+from tests.tiny import TINY_A, TINY_B, TINY_C, make_weights_dict
 
 
 def test_rms_norm_is_library_rms_norm():
@@ -391,3 +391,33 @@ def test_last_logits_row_and_greedy_rollout_agree_with_prefix_recomputation():
     out = P.greedy_generate(w, cfg, prompt, 40)
     full = P.forward(w, cfg, prompt + out)
     assert [int(full[len(prompt) - 1 + i].argmax()) for i in range(40)] == out
+
+
+@pytest.mark.parametrize("tiny", [TINY_B, TINY_C], ids=["B", "C"])
+def test_attention_block_splits_heads_row_block_by_row_block_and_joins_them_head_major(tiny):
+    """With ``o_proj`` set to select the D columns of query head j, the block's output is the
+    library's attention of that head alone: q from rows [jD, (j+1)D) of ``q_proj``, k and v from
+    rows [gD, (g+1)D) of ``k_proj`` / ``v_proj`` with g = j // (heads per kv head), each after the
+    library's ``rms_norm`` over D and the rotation pinned above.  A head split taken from the wrong
+    axis (interleaved heads), a kv head map j % nkv, or a concat that is not head-major fails it."""
+    c = tiny["config"]
+    nq, nkv, d, hid = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"], c["hidden_size"]
+    cfg = dict(num_heads=nq, num_kv_heads=nkv, head_dim=d, rms_norm_eps=c["rms_norm_eps"], rope_theta=c["rope_theta"])
+    w = {k.replace("model.layers.0.self_attn", "p"): v.double() for k, v in make_weights_dict(tiny).items()
+         if k.startswith("model.layers.0.self_attn")}
+    t = 11
+    g = torch.Generator().manual_seed(44)
+    x = torch.randn(t, hid, generator=g, dtype=torch.float64)
+    pos = torch.arange(t) + 3
+    cos, sin = P.rope_cos_sin(d, c["rope_theta"], pos, torch.float64)
+    for j in range(nq):
+        kv = j // (nq // nkv)
+        select = torch.zeros(d, nq * d, dtype=torch.float64)
+        select[torch.arange(d), j * d + torch.arange(d)] = 1.0
+        out = P.attention_block(dict(w, **{"p.o_proj.weight": select}), "p", cfg, x, pos)
+        q = F.rms_norm(x @ w["p.q_proj.weight"][j * d:(j + 1) * d].T, (d,), w["p.q_norm.weight"], c["rms_norm_eps"])
+        k = F.rms_norm(x @ w["p.k_proj.weight"][kv * d:(kv + 1) * d].T, (d,), w["p.k_norm.weight"], c["rms_norm_eps"])
+        v = x @ w["p.v_proj.weight"][kv * d:(kv + 1) * d].T
+        q, k = P.apply_rope(q[None], cos, sin), P.apply_rope(k[None], cos, sin)
+        ref = F.scaled_dot_product_attention(q[None], k[None], v[None, None], is_causal=True)[0, 0]
+        torch.testing.assert_close(out, ref, rtol=1e-9, atol=1e-9)

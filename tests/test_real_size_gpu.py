@@ -4,7 +4,13 @@ sizes: hidden 5120, 64/8 heads, so that heads * head size = 8192 is not the widt
 25600) with two layers of random weights: the 32-bit path and the bfloat16
 path against the plain implementation, whole, token by token, in portions and mixed.  These are
 the sizes at which the kernels' wide paths run (16-byte norm loads, the streaming matrix
-product's real shapes, a vocabulary that is no power of two, the 128-wide MFMA attention)."""
+product's real shapes, a vocabulary that is no power of two, the 128-wide MFMA attention).
+
+Then the shapes that the measurement program times, again against the plain implementation:
+decode-only steps of 8, 24 and 64 requests behind prompts of about 1,024 tokens, recorded and
+replayed and started ahead of their tokens; one prompt of 2,048 tokens whole, cut, and behind a
+prefix taken from the cache; contexts of 8,300 and 20,000 tokens on a narrow model with the real
+head geometry.  The plain implementation runs on the GPU here, in torch's exact float32."""
 import numpy as np
 import pytest
 import torch
@@ -23,47 +29,72 @@ CONFIG_14B = dict(CONFIG, hidden_size=5120, num_attention_heads=40, intermediate
 # 8 query heads per kv head; the attention's output is wider than the model (8192 against 5120), the
 # feed-forward's inner size is beyond what one block keeps of x: further branches of the products' plans
 CONFIG_32B = dict(CONFIG, hidden_size=5120, num_attention_heads=64, intermediate_size=25600)
+# the real head geometry (4 query heads of 128 per kv head, page 16) on a narrow model: long contexts stay cheap
+CONFIG_NARROW = dict(CONFIG, hidden_size=512, num_attention_heads=8, num_key_value_heads=2, intermediate_size=1536,
+                     vocab_size=3000)
+
+
+class Sized:
+    """Random weights of one configuration on the GPU (rounded through bfloat16 like a stored
+    checkpoint): bound models of either type, and the plain implementation's float copy."""
+
+    def __init__(self, config, seed=0):
+        from jax_vllm_amd.config import resolve
+        from jax_vllm_amd.parts import DecoderModel
+        from jax_vllm_amd.weights.random_init import _draw
+
+        P.use_exact_float32_products()
+        arch, cfg, _ = resolve(config)
+        self.cfg, self.spec = cfg, arch.build_spec(cfg)
+        self.names = DecoderModel(self.spec).tensor_specs()
+        self.dev = {n: _draw(ts, seed, n, 0.02, 0.02, device="cuda").to(torch.bfloat16) for n, ts in self.names.items()}
+        self.plain_w = {n: t.float() for n, t in self.dev.items()}
+        self.plain_cfg = dict(
+            vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size,
+            num_hidden_layers=cfg.num_hidden_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads,
+            head_dim=cfg.head_dim, rms_norm_eps=cfg.rms_norm_eps, rope_theta=cfg.rope_theta,
+            tie_word_embeddings=cfg.tie_word_embeddings)
+        self._models = {}
+
+    def model(self, dtype):
+        from jax_vllm_amd.parts import DecoderModel
+        from jax_vllm_amd.weights.loader import target_dtype
+
+        if dtype not in self._models:
+            compute = torch.float32 if dtype == "float32" else torch.bfloat16
+            m = DecoderModel(self.spec)
+            m.bind({n: self.dev[n].to(target_dtype(self.names[n].role, compute)).contiguous() for n in self.names}, compute)
+            self._models[dtype] = m
+        return self._models[dtype]
+
+    def plain(self, tokens, rows=None) -> np.ndarray:
+        return P.forward(self.plain_w, self.plain_cfg, tokens, rows=rows).cpu().numpy()
 
 
 @pytest.fixture(scope="module", params=[CONFIG, CONFIG_14B, CONFIG_32B], ids=["8b", "14b", "32b"])
 def big(request):
-    CONFIG = request.param
-    from jax_vllm_amd.config import resolve
-    from jax_vllm_amd.parts import DecoderModel
-    from jax_vllm_amd.weights.random_init import _draw
-
-    arch, cfg, _ = resolve(CONFIG)
-    spec = arch.build_spec(cfg)
-    names = DecoderModel(spec).tensor_specs()
-    dev = {n: _draw(ts, 0, n, 0.02, 0.02, device="cuda").to(torch.bfloat16) for n, ts in names.items()}
-    plain_w = {n: t.float().cpu() for n, t in dev.items()}
-    plain_cfg = dict(vocab_size=cfg.vocab_size, hidden_size=cfg.hidden_size, intermediate_size=cfg.intermediate_size,
-                     num_hidden_layers=cfg.num_hidden_layers, num_heads=cfg.num_heads, num_kv_heads=cfg.num_kv_heads,
-                     head_dim=cfg.head_dim, rms_norm_eps=cfg.rms_norm_eps, rope_theta=cfg.rope_theta,
-                     tie_word_embeddings=cfg.tie_word_embeddings)
+    sized = Sized(request.param)
     rng = np.random.default_rng(0)
-    reqs = {f"r{i}": rng.integers(0, cfg.vocab_size, size=n).tolist() for i, n in enumerate((64, 150, 300, 97))}
-    torch.set_num_threads(16)
-    want = {r: P.forward(plain_w, plain_cfg, t).numpy() for r, t in reqs.items()}
-
-    def model(dtype):
-        from jax_vllm_amd.weights.loader import target_dtype
-
-        compute = torch.float32 if dtype == "float32" else torch.bfloat16
-        m = DecoderModel(spec)
-        m.bind({n: dev[n].to(target_dtype(names[n].role, compute)).contiguous() for n in names}, compute)
-        return m
-
-    return model, reqs, want
+    reqs = {f"r{i}": rng.integers(0, sized.cfg.vocab_size, size=n).tolist() for i, n in enumerate((64, 150, 300, 97))}
+    want = {r: sized.plain(t) for r, t in reqs.items()}
+    if request.param is CONFIG:
+        # the oracle on the GPU is the oracle on the CPU: same formulas, exact float32 products
+        on_cpu = P.forward({n: t.cpu() for n, t in sized.plain_w.items()}, sized.plain_cfg, reqs["r0"]).numpy()
+        scale = float(np.abs(on_cpu).max())
+        assert float(np.abs(on_cpu - want["r0"]).max()) <= 1e-5 * scale
+    yield sized.model, reqs, want
+    del sized
+    torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_real_layer_sizes_every_cut(big, dtype):
+def every_cut(core, reqs, want, dtype, check_logits=check_logits) -> float:
+    """Each request whole; one with its last 32 tokens one by one; all four in portions of changing
+    size beside single tokens of the others.  Returns the largest error seen, as a fraction of the
+    largest logit."""
     from jax_vllm_amd.engine.entries import StepEntry
 
-    model, reqs, want = big
-    core = make_core(None, dtype, 16, pages=48, seqs=4, model=model(dtype), graphs=(dtype == "bfloat16"))
     scale = max(float(np.abs(w).max()) for w in want.values())
+    errs = []
 
     def run(entries):
         out = core.run([StepEntry(r, t, range(len(t))) for r, t in entries]).cpu().numpy()
@@ -76,14 +107,14 @@ def test_real_layer_sizes_every_cut(big, dtype):
     # whole, then most of it in one step and the last 32 tokens one by one
     for r, toks in reqs.items():
         core.start_request(r)
-        check_logits(dtype, run([(r, toks)])[0], want[r], scale, f"{r} whole")
+        errs.append(check_logits(dtype, run([(r, toks)])[0], want[r], scale, f"{r} whole"))
         core.finish_request(r)
     r, toks = "r1", reqs["r1"]
     core.start_request(r)
     got = run([(r, toks[:-32])])
     for i in range(len(toks) - 32, len(toks)):
         got += run([(r, toks[i:i + 1])])
-    check_logits(dtype, np.concatenate(got), want[r], scale, f"{r} tail one by one")
+    errs.append(check_logits(dtype, np.concatenate(got), want[r], scale, f"{r} tail one by one"))
     core.finish_request(r)
     # portions of changing size beside single tokens of other requests, pages taken again
     fed = {r: 0 for r in reqs}
@@ -99,6 +130,205 @@ def test_real_layer_sizes_every_cut(big, dtype):
             fed[r] += len(t)
     for r in reqs:
         assert fed[r] == len(reqs[r])
-        check_logits(dtype, np.concatenate(got[r]), want[r], scale, f"{r} mixed")
+        errs.append(check_logits(dtype, np.concatenate(got[r]), want[r], scale, f"{r} mixed"))
         core.finish_request(r)
+    core.cache.check_invariants()
+    return max(errs) / scale
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_real_layer_sizes_every_cut(big, dtype):
+    model, reqs, want = big
+    # replayed steps here are those of one row (the tail one by one); more rows: the tests of the benchmark's shapes below
+    core = make_core(None, dtype, 16, pages=48, seqs=4, model=model(dtype), graphs=(dtype == "bfloat16"))
+    every_cut(core, reqs, want, dtype)
+
+
+def test_all_36_layers_of_the_8b_sizes_every_cut(capsys):
+    """The whole depth of the configuration that the measurement program runs, once: 36 layers of
+    the 8B sizes, 4 prompts of 64 to 300 tokens, whole / last 32 tokens one by one / portions /
+    mixed.  Rounding errors add up like a random walk over the layers (measured against the plain
+    implementation in float64, as a fraction of the largest logit: the plain float32 implementation
+    itself 0.5e-5 at 2 layers, 1.4e-5 at 12, 2.2e-5 at 36; the 32-bit engine 0.6e-5, 1.3e-5, 2.3e-5;
+    the bfloat16 engine 1.2e-2, 2.6e-2, 4.4e-2 with cosines from 0.9999 down to 0.9988), so at this
+    depth the oracle is the float64 one and the bounds are: 32-bit engine 4e-5 and at most twice the
+    plain float32 implementation's own error; bfloat16 engine 6e-2 and cosine 0.998 (the bar of the
+    reference's own bfloat16 test, tests/test_parity.py:26-29 there)."""
+    sized = Sized(dict(CONFIG, num_hidden_layers=36))
+    rng = np.random.default_rng(0)
+    reqs = {f"r{i}": rng.integers(0, sized.cfg.vocab_size, size=n).tolist() for i, n in enumerate((64, 150, 300, 97))}
+    w64 = {n: t.double() for n, t in sized.plain_w.items()}
+    want = {r: P.forward(w64, sized.plain_cfg, t).cpu().numpy() for r, t in reqs.items()}
+    del w64
+    scale = max(float(np.abs(w).max()) for w in want.values())
+    plain32 = max(float(np.abs(sized.plain(t) - want[r]).max()) for r, t in reqs.items())
+    assert plain32 <= 3e-5 * scale
+
+    def deep_check(dtype, got, want, scale=None, what=""):
+        err = float(np.abs(np.asarray(got, dtype=np.float64) - want).max())
+        if dtype == "float32":
+            assert err <= 4e-5 * scale and err <= 2 * plain32, f"{what}: max error {err} (scale {scale}, plain float32 {plain32})"
+        else:
+            assert err <= 6e-2 * scale, f"{what}: max error {err} (scale {scale})"
+            g, w = np.asarray(got, dtype=np.float64), want
+            cos = (g * w).sum(-1) / (np.linalg.norm(g, axis=-1) * np.linalg.norm(w, axis=-1) + 1e-30)
+            assert cos.min() >= 0.998, f"{what}: cosine {cos.min()}"
+        return err
+
+    for dtype in ("float32", "bfloat16"):
+        core = make_core(None, dtype, 16, pages=48, seqs=4, model=sized.model(dtype), graphs=True)
+        err = every_cut(core, reqs, want, dtype, check_logits=deep_check)
+        with capsys.disabled():
+            print(f"\n[36 layers, {dtype}] largest error / largest logit = {err:.3e} (plain float32: {plain32 / scale:.3e})",
+                  flush=True)
+        del core
+        sized._models.clear()
+        torch.cuda.empty_cache()
+
+
+# ------------------------------------------------------------------ the shapes that the measurement program times
+@pytest.fixture(scope="module")
+def sized_8b():
+    sized = Sized(CONFIG)
+    yield sized
+    del sized
+    torch.cuda.empty_cache()
+
+
+DECODE_STEPS = 12
+
+
+@pytest.mark.parametrize("dtype,batch", [("bfloat16", 8), ("bfloat16", 24), ("bfloat16", 64), ("float32", 8), ("float32", 24), ("float32", 64)])
+def test_decode_steps_of_many_requests_behind_long_prompts_replayed_and_started_ahead(sized_8b, dtype, batch):
+    """What the decode benchmark times: ``batch`` requests behind prompts of 1,000 to 1,060 tokens
+    (prefilled under a budget of 2,048 tokens a step), then decode-only steps of all of them,
+    recorded, replayed and started ahead of their tokens.  First through the entry point: every
+    token must be the plain implementation's choice.  Then the same kind of steps through the step
+    function with given tokens: every row's logits against the plain ones."""
+    from jax_vllm_amd.engine.entries import StepEntry
+    from jax_vllm_amd.engine.llm import LLM
+    from jax_vllm_amd.engine.request import SamplingParams
+
+    sized = sized_8b
+    vocab = sized.cfg.vocab_size
+    rng = np.random.default_rng(100 + batch)
+    lens = rng.integers(1000, 1061, size=batch).tolist()
+    prompts = [rng.integers(0, vocab, size=n).tolist() for n in lens]
+    llm = LLM(sized.model(dtype), dtype=dtype, max_num_seqs=batch, max_model_len=1280, max_num_batched_tokens=2048,
+              block_size=16, use_hip_graphs=True, decode_ahead=True, enable_prefix_cache=False)
+    rids = [llm.add_request(p, SamplingParams(max_new_tokens=200)) for p in prompts]
+    outs = {r: [] for r in rids}
+
+    def step():
+        events = llm.step()
+        for e in events:
+            outs[e.request_id].append(e.token)
+        return len(events)
+
+    # as the measurement does: prompts two a step beside the decodes of those that are through, untimed there ...
+    while llm.scheduler.waiting or any(r.num_remaining > 1 or not r.output_ids for r in llm.scheduler.running):
+        step()
+    before = (llm.stats.graph_replays, llm.stats.steps_ahead)
+    for _ in range(DECODE_STEPS):            # ... then the steps it times: one token of every request
+        assert step() == batch
+    assert llm.stats.graph_replays - before[0] >= DECODE_STEPS - 2 and llm.stats.steps_ahead - before[1] >= DECODE_STEPS - 2
+    assert llm.stats.preemptions == 0
+    llm.abort_all()
+    tight = dtype == "float32"
+    for i, (p, rid) in enumerate(zip(prompts, rids)):
+        out = outs[rid]
+        assert len(out) >= DECODE_STEPS + 1
+        rows = list(range(len(p) - 1, len(p) + len(out) - 1))
+        logits = sized.plain(p + out[:-1], rows)
+        for k, t in enumerate(out):
+            margin = float(logits[k].max() - logits[k][t])
+            allowed = (1e-4 if tight else 0.04) * float(np.abs(logits[k]).max())
+            assert margin <= allowed, f"request {i}, token {k}: engine's {t} is {margin} below the plain maximum"
+
+    # the step function itself, with given tokens, so that every row's logits can be compared
+    core = llm.core
+    assert not core.cache.requests
+    replays_before = core.graph_replays
+    tails = [rng.integers(0, vocab, size=DECODE_STEPS).tolist() for _ in range(batch)]
+    ids = [f"q{i}" for i in range(batch)]
+    got = {r: [] for r in ids}
+    for r in ids:
+        core.start_request(r)
+    for first in range(0, batch, 2):         # two prompts a step: about 2,048 tokens
+        pair = list(range(first, min(first + 2, batch)))
+        out = core.run([StepEntry(ids[i], prompts[i], [len(prompts[i]) - 1]) for i in pair]).cpu().numpy()
+        for k, i in enumerate(pair):
+            got[ids[i]].append(out[k:k + 1])
+    for step in range(DECODE_STEPS):
+        out = core.run([StepEntry(ids[i], [tails[i][step]], [0]) for i in range(batch)]).cpu().numpy()
+        for i in range(batch):
+            got[ids[i]].append(out[i:i + 1])
+    assert core.graph_replays - replays_before >= DECODE_STEPS - 1
+    scale = None
+    for i in range(batch):
+        rows = list(range(lens[i] - 1, lens[i] + DECODE_STEPS))
+        want = sized.plain(prompts[i] + tails[i], rows)
+        scale = scale or float(np.abs(want).max())
+        check_logits(dtype, np.concatenate(got[ids[i]]), want, scale, f"request {i} of {batch}")
+        core.finish_request(ids[i])
+    core.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_of_2048_tokens_whole_cut_and_behind_a_cached_prefix(sized_8b, dtype):
+    """What the prefill benchmark times: one prompt of 2,048 tokens in one step; the same prompt as
+    1,500 + 548; and a second prompt that shares its first 1,504 tokens, which are then found in
+    the cache, so that only 544 tokens run, behind pages that another request wrote.  Logits at 64
+    places spread over the prompt (page and tile edges among them)."""
+    from jax_vllm_amd.engine.entries import StepEntry
+
+    sized = sized_8b
+    rng = np.random.default_rng(7)
+    n = 2048
+    prompt = rng.integers(0, sized.cfg.vocab_size, size=n).tolist()
+    rows = sorted(set(np.linspace(0, n - 1, 50).astype(int).tolist()
+                      + [1, 15, 16, 63, 64, 127, 128, 1023, 1024, 1499, 1500, 1501, 1503, 1504, 1505, 2046]))[:64]
+    assert len(rows) == 64
+    want = sized.plain(prompt, rows)
+    scale = float(np.abs(want).max())
+    core = make_core(None, dtype, 16, pages=400, seqs=3, model=sized.model(dtype), prefix=True)
+    core.start_request("whole", prompt)
+    check_logits(dtype, core.run([StepEntry("whole", prompt, rows)]).cpu().numpy(), want, scale, "whole")
+    # the pages of "whole" are hashed now; a request that is started without its prompt does not look for them
+    core.start_request("cut")
+    first = [r for r in rows if r < 1500]
+    got = [core.run([StepEntry("cut", prompt[:1500], first)]).cpu().numpy(),
+           core.run([StepEntry("cut", prompt[1500:], [r - 1500 for r in rows if r >= 1500])]).cpu().numpy()]
+    check_logits(dtype, np.concatenate(got), want, scale, "1,500 + 548")
+    other = prompt[:1504] + rng.integers(0, sized.cfg.vocab_size, size=n - 1504).tolist()
+    assert core.start_request("behind", other) == 1504
+    late = [r for r in rows if r >= 1504]
+    got = core.run([StepEntry("behind", other[1504:], [r - 1504 for r in late])]).cpu().numpy()
+    check_logits(dtype, got, sized.plain(other, late), scale, "544 behind 1,504 cached")
+    for r in ("whole", "cut", "behind"):
+        core.finish_request(r)
+    core.cache.check_invariants()
+
+
+@pytest.mark.parametrize("dtype,length", [("float32", 8300), ("bfloat16", 8300), ("bfloat16", 20000)])
+def test_long_contexts_with_the_real_head_geometry(dtype, length):
+    """One request of 8,300 (20,000) tokens in portions of 2,048, then 32 tokens one by one (replayed
+    steps), on a narrow model with heads of 128, 4 per kv head, pages of 16: every position's logits."""
+    from jax_vllm_amd.engine.entries import StepEntry
+
+    sized = Sized(CONFIG_NARROW, seed=5)
+    rng = np.random.default_rng(length)
+    toks = rng.integers(0, sized.cfg.vocab_size, size=length + 32).tolist()
+    want = sized.plain(toks)
+    core = make_core(None, dtype, 16, pages=-(-(length + 32) // 16) + 2, seqs=2, model=sized.model(dtype), graphs=True)
+    core.start_request("a")
+    got = []
+    for at in range(0, length, 2048):
+        part = toks[at:min(at + 2048, length)]
+        got.append(core.run([StepEntry("a", part, range(len(part)))]).cpu().numpy())
+    for i in range(length, length + 32):
+        got.append(core.run([StepEntry("a", toks[i:i + 1], [0])]).cpu().numpy())
+    assert core.graph_replays >= 30
+    check_logits(dtype, np.concatenate(got), want, what=f"{length} tokens")
+    core.finish_request("a")
     core.cache.check_invariants()
