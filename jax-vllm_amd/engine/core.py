@@ -153,8 +153,7 @@ class EngineCore:
             for w in e.want:
                 if not 0 <= int(w) < len(e.tokens):
                     raise ValueError(f"request {e.request_id!r}: wanted place {w} outside its {len(e.tokens)} tokens")
-        for e in entries:
-            self.cache.reserve(e.request_id, len(e.tokens))
+        self._reserve_all([(e.request_id, len(e.tokens)) for e in entries])
         self._zero_new_state()
         if self._graphable(entries):
             logits = self._run_decode_graph(entries)
@@ -166,6 +165,21 @@ class EngineCore:
         for e in entries:
             self.cache.commit(e.request_id, e.tokens)
         return logits
+
+    def _reserve_all(self, needs) -> None:
+        """Pages for every (request, new tokens) of a step, or ``OutOfPages`` with no table changed:
+        the pools are asked for the sum first, so an entry that does not fit never leaves the
+        entries before it with pages they did not have."""
+        from ..cache.page_pool import OutOfPages
+
+        cache = self.cache
+        promised = [0] * len(self.group_keys)
+        for rid, n in needs:
+            if not cache.can_store(rid, n, reserve=promised):
+                raise OutOfPages(f"request {rid!r}: no pages for {n} more token(s) beside the step's other entries")
+            promised = [p + k for p, k in zip(promised, cache.pages_needed(rid, n))]
+        for rid, n in needs:
+            cache.reserve(rid, n)
 
     # ---- decode-only steps as replayed HIP graphs
     def _graphable(self, entries) -> bool:
@@ -194,13 +208,12 @@ class EngineCore:
         g = self._graphs.get(self._graph_key(request_ids, 1))
         if g is None or g.graph is None:
             return None
-        promised = [0] * len(self.group_keys)
-        for r in request_ids:
-            if not cache.can_store(r, 1, reserve=promised):
-                return None
-            promised = [p + n for p, n in zip(promised, cache.pages_needed(r, 1))]
-        for r in request_ids:
-            cache.reserve(r, 1)
+        from ..cache.page_pool import OutOfPages
+
+        try:
+            self._reserve_all([(r, 1) for r in request_ids])
+        except OutOfPages:
+            return None
         self.steps_followed += 1
         return self._run_decode_graph([StepEntry(r, [0], [0]) for r in request_ids], token_source)
 
@@ -253,6 +266,12 @@ class EngineCore:
                 if sig[i] is not None:
                     bt[i, :] = 0
                     sig[i] = None
+        if r < rb:
+            # rows that pad the step write the spare state row: it starts from zero in every step, so
+            # that a mixer which keeps adding to its state never runs it up to infinity there
+            for m in self.memories:
+                if m.state is not None:
+                    m.state[self._spare_slot].zero_()
         g.dev.copy_(g.host_tensor, non_blocking=True)
         if g.copied is None:
             g.copied = torch.cuda.Event()

@@ -31,29 +31,43 @@ class Sampler:
         self.device = device
         self._host, self._turn = [], 0
 
-    def _pinned(self, rows: int) -> torch.Tensor:
+    def _pinned(self, rows: int) -> dict:
+        """The next set of pinned host buffers (token ids back, temperatures and keys out).  A set is
+        used again only after ``HOST_BUFFERS`` further launches, and a launch is finished (its event
+        awaited) before the launch after the next one starts, so no copy is still reading or
+        writing it."""
         if len(self._host) < self.HOST_BUFFERS:
-            self._host.append(torch.empty(max(rows, 64), dtype=torch.int32, pin_memory=True))
+            self._host.append(None)
         self._turn = (self._turn + 1) % len(self._host)
-        if self._host[self._turn].numel() < rows:
-            self._host[self._turn] = torch.empty(rows, dtype=torch.int32, pin_memory=True)
-        return self._host[self._turn]
+        have = self._host[self._turn]
+        if have is None or have["tokens"].numel() < rows:
+            n = max(rows, 64)
+            have = self._host[self._turn] = {
+                "tokens": torch.empty(n, dtype=torch.int32, pin_memory=True),
+                "temperature": torch.empty(n, dtype=torch.float32, pin_memory=True),
+                "keys": torch.empty(n, dtype=torch.int64, pin_memory=True),
+            }
+        return have
 
     def launch(self, logits: torch.Tensor, temperatures: Sequence[float], keys: Sequence[int]) -> Drawn:
         """Start choosing one token id per row of ``logits`` [M, V] (float32, on the device) and copying
         them to the host; nothing here waits for the GPU."""
         m = logits.shape[0]
+        host = self._pinned(m)
         if all(t <= 0.0 for t in temperatures):
             out = K.sample(logits)
         else:
-            temp = torch.tensor(list(temperatures), dtype=torch.float32, device=self.device)
-            key = torch.tensor(list(keys), dtype=torch.int64, device=self.device)
+            # through pinned memory and without waiting: a copy from pageable memory would hold the host
+            # until the logits are there, and the step after this one could not be started ahead
+            host["temperature"][:m] = torch.as_tensor(list(temperatures), dtype=torch.float32)
+            host["keys"][:m] = torch.as_tensor(list(keys), dtype=torch.int64)
+            temp = host["temperature"][:m].to(self.device, non_blocking=True)
+            key = host["keys"][:m].to(self.device, non_blocking=True)
             out = K.sample(logits, temp, key)
-        host = self._pinned(m)
-        host[:m].copy_(out, non_blocking=True)
+        host["tokens"][:m].copy_(out, non_blocking=True)
         copied = torch.cuda.Event()
         copied.record()
-        return Drawn(out, host, copied, m, logits.shape[1])
+        return Drawn(out, host["tokens"], copied, m, logits.shape[1])
 
     def finish(self, drawn: Drawn) -> list:
         """The token ids of a ``launch``, once they are there."""

@@ -34,6 +34,12 @@ def test_embedding(dtype, hidden, vocab):
     h = torch.empty(5, hidden, dtype=torch.float32).cuda()
     K().embedding(h, table, ids)
     torch.testing.assert_close(h, table[ids.long()].float(), rtol=0, atol=0)
+    # an id that no row has (the sampling kernel's answer for a row of logits without a maximum is the
+    # vocabulary size) reads nothing: its row is NaN, the other rows are untouched by it
+    bad = torch.tensor([3, vocab, -1, 2 ** 31 - 1, 1], dtype=torch.int32).cuda()
+    K().embedding(h, table, bad)
+    assert torch.isnan(h[1:4]).all()
+    torch.testing.assert_close(h[[0, 4]], table[[3, 1]].float(), rtol=0, atol=0)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
