@@ -81,10 +81,12 @@ def measure_decode(llm, batch, steps, warmup, rng, vocab, prompt_len=PROMPT_LEN)
 
 
 def measure_prefill(llm, rng, vocab, repeats=3):
+    """Seconds of one 2,048-token prompt through the step function: the median of ``repeats`` runs
+    after one that warms up."""
     from jax_vllm_amd.engine.entries import StepEntry
 
     core = llm.core
-    best = None
+    times = []
     for i in range(repeats + 1):
         toks = rng.integers(0, vocab, size=PREFILL_TOKENS).tolist()
         rid = f"prefill{i}"
@@ -96,8 +98,98 @@ def measure_prefill(llm, rng, vocab, repeats=3):
         dt = time.perf_counter() - t0
         core.finish_request(rid)
         if i > 0:  # the first run warms up
-            best = dt if best is None else min(best, dt)
-    return best
+            times.append(dt)
+    return sorted(times)[len(times) // 2]
+
+
+KERNEL_GROUPS = (          # substring of a kernel's name -> what it is counted as
+    ("gemm_skinny", "products_own"), ("gemm_tile64", "products_own"), ("gemm_rows", "products_own"),
+    ("gemm_f32", "products_own"),
+    ("Cijk", "products_library"), ("rocblas", "products_library"), ("hipblaslt", "products_library"),
+    ("attn_", "attention"), ("paged_attention", "attention"),
+    ("add_rmsnorm", "norm_residual"), ("add_parts", "norm_residual"), ("rmsnorm", "norm_residual"),
+    ("qk_norm_rope", "rope_kv_write"), ("rope_table", "rope_kv_write"), ("v_pages_write", "rope_kv_write"),
+    ("gated_mul", "activation"), ("embedding", "embedding"), ("sample_", "sampling"), ("add_bias", "bias"),
+)
+
+
+def kernel_shares(run) -> dict:
+    """Share of the GPU's kernel time by kind of kernel while ``run()`` executes (torch's profiler over
+    the HIP activity records; kernels of replayed graphs are seen too)."""
+    import torch
+    from torch.profiler import ProfilerActivity, profile
+
+    sync()
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        run()
+        sync()
+    totals = {}
+    for e in prof.key_averages():
+        t = float(getattr(e, "self_device_time_total", 0.0))
+        if t <= 0.0 or str(e.device_type).endswith("CPU"):
+            continue
+        group = next((g for key, g in KERNEL_GROUPS if key in e.key), "other")
+        totals[group] = totals.get(group, 0.0) + t
+    whole = sum(totals.values()) or 1.0
+    return {g: round(t / whole, 4) for g, t in sorted(totals.items(), key=lambda kv: -kv[1])}
+
+
+def calibrate(device="cuda") -> dict:
+    """What a plain streaming read and a plain matrix-core loop reach on this box: GB/s of a kernel that
+    only reads (8 buffers of 201 MB in turn, the size of one gate/up weight: nothing comes from a cache)
+    and TFLOP/s of a kernel that only issues bf16 MFMA on registers."""
+    import torch
+
+    from jax_vllm_amd.ops import kernels as K
+
+    sink = torch.zeros(4, dtype=torch.float32, device=device)
+    nbytes = 2 * 12288 * 4096 * 2
+    buffers = [torch.zeros(nbytes // 2, dtype=torch.bfloat16, device=device) for _ in range(8)]
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for b in buffers:
+        K.calibrate_read(b, sink)
+    sync()
+    start.record()
+    for _ in range(4):
+        for b in buffers:
+            K.calibrate_read(b, sink)
+    end.record()
+    sync()
+    read_gbs = 32 * nbytes / (start.elapsed_time(end) * 1e-3) / 1e9
+    blocks, turns = 256 * 8, 4096
+    K.calibrate_mfma(sink, turns, blocks)
+    sync()
+    start.record()
+    flops = sum(K.calibrate_mfma(sink, turns, blocks) for _ in range(4))
+    end.record()
+    sync()
+    tflops = flops / (start.elapsed_time(end) * 1e-3) / 1e12
+    del buffers
+    return {"hbm_read_gbs": round(read_gbs, 1), "hbm_read_frac_of_peak": round(read_gbs / PEAK_HBM_GBS, 4),
+            "mfma_bf16_tflops": round(tflops, 1), "mfma_frac_of_peak": round(tflops * 1e12 / PEAK_FLOPS["bf16"], 4)}
+
+
+def measure_ttft(llm, rng, vocab, prompt_len=2048, shared=1024):
+    """Time to the first token of a prompt, cold (nothing of it in the cache) and warm (its first
+    ``shared`` tokens were another request's prompt prefix and are taken from the cache); the
+    reference's harness measures this pair over HTTP (scripts/bench_vllm.py:728-789)."""
+    from jax_vllm_amd import SamplingParams
+
+    one = SamplingParams(max_new_tokens=1)
+    llm.generate([rng.integers(0, vocab, size=prompt_len).tolist()], one)      # warms the kernels, shares nothing
+    prefix = rng.integers(0, vocab, size=shared).tolist()
+    out = {}
+    for name in ("cold", "warm"):
+        prompt = prefix + rng.integers(0, vocab, size=prompt_len - shared).tolist()
+        hits = llm.stats.cache_hit_tokens
+        sync()
+        t0 = time.perf_counter()
+        llm.generate([prompt], one)
+        sync()
+        out[f"{name}_ttft_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
+        out[f"{name}_cache_hit_tokens"] = llm.stats.cache_hit_tokens - hits
+    out.update(prompt_len=prompt_len, shared_prefix=shared)
+    return out
 
 
 def measure_long_prompt(llm, rng, vocab, prompt_len):
@@ -169,10 +261,13 @@ def main():
                     help="run only the first layers of the shape's (both numbers are reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="measure the headline batch only")
-    ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt"], default=None,
+    ap.add_argument("--no-kernel-share", action="store_true", help="leave out the per-kernel time shares")
+    ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt", "ttft", "calibrate"], default=None,
                     help="run one phase alone and print its result (for profiling); mixed: 32 running decodes "
                          "joined by 4 prompts of 3,000 tokens in portions of 512 under a budget of 2,048; "
-                         "long-prompt: one prompt of --prompt-len tokens (default 32,768) in portions of 2,048")
+                         "long-prompt: one prompt of --prompt-len tokens (default 32,768) in portions of 2,048; "
+                         "ttft: time to first token of a 2,048-token prompt, cold and with its first 1,024 tokens "
+                         "in the cache; calibrate: the plain read and matrix-core rates of this box")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--prompt-len", type=int, default=None,
                     help="with --only decode: prompt length of the decoding requests (long-context runs, default "
@@ -198,6 +293,16 @@ def main():
     rng = np.random.default_rng(0)
     max_batch = args.batch if (args.skip_points or args.only) else max(64, args.batch)
     block = 16
+    if args.only == "calibrate":
+        print(json.dumps(calibrate()), flush=True)
+        return
+    if args.only == "ttft":
+        llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=4, max_model_len=4096,
+                  num_blocks=1 + 4 * (4096 // block), max_num_batched_tokens=2048, enable_prefix_cache=True)
+        res = measure_ttft(llm, rng, vocab)
+        res.update(model=model_name, layers=layers)
+        print(json.dumps(res), flush=True)
+        return
     if args.only == "mixed":
         llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=36, max_model_len=8192,
                   num_blocks=1 + 32 * (4608 // block) + 4 * (3200 // block), max_num_batched_tokens=2048,
@@ -241,17 +346,43 @@ def main():
     tps, step_s, mean_ctx = measure_decode(llm, args.batch, args.steps, args.warmup, rng, vocab)
     read_bytes = wbytes + args.batch * mean_ctx * kv_per_token
     achieved = read_bytes / step_s / 1e9
-    points = {}
+    points, detail = {}, {}
     if not args.skip_points:
-        for b in (1, 64):
-            n = min(args.steps, 128)
-            points[f"decode_b{b}"] = round(measure_decode(llm, b, n, min(args.warmup, 8), rng, vocab)[0], 1)
+        n = min(args.steps, 128)
+        # batch 1 and 64 from 1,024-token prompts; batch 8 near the benchmark context of 8,192 tokens
+        for name, b, plen, k in (("decode_b1", 1, PROMPT_LEN, n), ("decode_b64", 64, PROMPT_LEN, n),
+                                 ("decode_b8_ctx8k", 8, 7900, min(n, 64))):
+            p_tps, p_step, p_ctx = measure_decode(llm, b, k, min(args.warmup, 8), rng, vocab, plen)
+            p_bytes = wbytes + b * p_ctx * kv_per_token
+            points[name] = round(p_tps, 1)
+            detail[name] = {"tok_s": round(p_tps, 1), "ms_per_step": round(p_step * 1e3, 4), "batch": b,
+                            "mean_context": round(p_ctx, 1), "gb_read": round(p_bytes / 1e9, 3),
+                            "frac": round(p_bytes / p_step / 1e9 / PEAK_HBM_GBS, 4)}
+    shares = None
+    if not args.no_kernel_share:
+        from jax_vllm_amd import SamplingParams
+        from jax_vllm_amd.engine.entries import StepEntry
+
+        for _ in range(args.batch):
+            llm.add_request(rng.integers(0, vocab, size=PROMPT_LEN).tolist(), SamplingParams(max_new_tokens=64))
+        while any(r.num_remaining > 1 or not r.output_ids for r in llm.scheduler.running) or llm.scheduler.waiting:
+            llm.step()
+        for _ in range(4):
+            llm.step()
+        shares = {"decode": kernel_shares(lambda: [llm.step() for _ in range(8)])}
+        llm.abort_all()
+        toks = rng.integers(0, vocab, size=PREFILL_TOKENS).tolist()
+        llm.core.start_request("share")
+        shares["prefill"] = kernel_shares(lambda: llm.core.run([StepEntry("share", toks, [PREFILL_TOKENS - 1])]))
+        llm.core.finish_request("share")
+    calibration = calibrate()
 
     line = {
         "metric": "decode_tokens_per_s", "value": round(tps, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
-        "data": "synthetic: seeded uniform-random token ids, random-init weights N(0,0.02), norms 1+N(0,0.02)",
+        "data": "synthetic: seeded uniform-random token ids, random-init weights N(0,0.02), norms 1+N(0,0.02); "
+                "prefill: median of 3 runs through the step function; decode: the whole engine",
         "config": {
             "model": model_name, "layers": layers, "layers_full": shape["num_hidden_layers"],
             "hidden": cfg["hidden_size"], "q_heads": nq, "kv_heads": cfg["num_key_value_heads"], "head_dim": d,
@@ -265,6 +396,9 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
         "points": points,
+        "points_detail": detail,
+        "calibration": calibration,
+        "kernel_share": shares,
     }
     print(json.dumps(line), flush=True)
 

@@ -762,3 +762,26 @@ def attn_decode_mfma(out, q, q_row_stride, k_pages, v_pages, block_tables, cu_se
                            _stream()),
         "attn_decode_mfma",
     )
+
+
+# --------------------------------------------------------------------------- what the chip delivers (for the measurement program)
+def calibrate_read(buffer: torch.Tensor, sink: torch.Tensor, blocks: int = 2048) -> None:
+    """Launch the kernel that only reads ``buffer`` (its byte size must split into 16-byte pieces
+    evenly over ``blocks`` blocks); time it from outside."""
+    _dev(buffer, sink)
+    _f32(sink, "sink")
+    n = buffer.numel() * buffer.element_size()
+    _need(n % 16 == 0 and (n // 16) % blocks == 0, f"{n} bytes do not split into 16-byte pieces over {blocks} blocks")
+    _check(library.core().jv_calibrate_read(_ptr(buffer), c_longlong(n), _ptr(sink), c_int(blocks), _stream()),
+           "calibrate_read")
+
+
+def calibrate_mfma(sink: torch.Tensor, turns: int, blocks: int) -> float:
+    """Launch the kernel that only issues bf16 matrix-core products on registers; returns the
+    floating-point operations it does."""
+    _dev(sink)
+    _f32(sink, "sink")
+    lib = library.core()
+    lib.jv_calibrate_mfma_flops.restype = ctypes.c_double
+    _check(lib.jv_calibrate_mfma(_ptr(sink), c_int(turns), c_int(blocks), _stream()), "calibrate_mfma")
+    return float(lib.jv_calibrate_mfma_flops(c_int(blocks), c_int(turns)))

@@ -40,5 +40,17 @@ def test_the_line_of_a_short_run_has_every_key():
     assert set(line["prefill"]) == {"value", "tokens", "ms", "frac"} and line["prefill"]["tokens"] == 2048
     assert line["roofline"]["bound"] == "hbm" and line["roofline"]["peak"] == 8000.0 and line["roofline"]["unit"] == "GB/s"
     assert abs(line["roofline"]["frac"] - line["roofline"]["achieved"] / 8000.0) < 1e-3
-    assert set(line["points"]) == {"decode_b1", "decode_b64"}
+    assert set(line["points"]) == {"decode_b1", "decode_b64", "decode_b8_ctx8k"}
+    assert all(isinstance(v, float) and v > 0 for v in line["points"].values())
+    for name, d in line["points_detail"].items():
+        assert set(d) == {"tok_s", "ms_per_step", "batch", "mean_context", "gb_read", "frac"} and d["tok_s"] == line["points"][name]
+        assert abs(d["frac"] - d["gb_read"] / (d["ms_per_step"] * 1e-3) / 8000.0) < 2e-3
+    assert line["points_detail"]["decode_b8_ctx8k"]["mean_context"] > 7900
+    assert "median of 3" in line["data"]
+    cal = line["calibration"]
+    assert 2000 < cal["hbm_read_gbs"] < 8000 and 500 < cal["mfma_bf16_tflops"] < 2600       # below the published peaks, above half-way off
+    for phase in ("decode", "prefill"):
+        shares = line["kernel_share"][phase]
+        assert abs(sum(shares.values()) - 1.0) < 0.01 and shares.get("attention", 0) > 0
+        assert shares.get("products_own", 0) + shares.get("products_library", 0) > 0.4
     assert abs(line["value"] - 8 / (line["ms_per_step"] * 1e-3)) < 0.01 * line["value"]
