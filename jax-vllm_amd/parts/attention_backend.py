@@ -82,6 +82,16 @@ def prefill_work_items(q_lens, context_lens, g: int, window: int, group_rows: in
     return [(r, a, b) for _, r, a, b in items]
 
 
+def pair_up_resident_items(items: list, first_round: int) -> list:
+    """For a launch whose blocks are all on the chip at once, two to a compute unit: the ``first_round`` heaviest
+    items (the blocks that get a unit to themselves at first) stay in descending order and the others follow in
+    ASCENDING order.  The hardware hands out blocks in the order of their numbers and comes back to the first unit
+    after one round, so the unit with the heaviest item gets the lightest one beside it (2,048 tokens, 32 q heads
+    over 8 kv heads of 128: 53.9 against 58.3 us; with more items than fit at once, heaviest first stays the
+    rule: 94.8 against 103.3 us at 3,072)."""
+    return items[:first_round] + items[first_round:][::-1]
+
+
 def prefill_item_shape(rows: int, nkv: int, group_rows: int, kernel_groups: int, compute_units: int,
                        waves_split: bool = False):
     """(groups per work item, whether light groups are paired with heavy ones) for a step with
@@ -112,6 +122,9 @@ def plan_mfma(ctx, nq: int, nkv: int, head_dim: int, window: int, device) -> Mfm
                                                   K.attn_prefill_waves_split(head_dim))
     prefill = prefill_work_items(ctx.q_lens_host, ctx.context_lens_host, g, window, group_rows, groups_per_item,
                                  balance=balance)
+    cus = K.compute_units(device)
+    if cus < len(prefill) * nkv <= RESIDENT_BLOCKS * cus:
+        prefill = pair_up_resident_items(prefill, cus // nkv)
     decode = [r for r, ql in enumerate(ctx.q_lens_host) if ql == 1]
     max_kv_decode = max([ctx.context_lens_host[r] + 1 for r in decode], default=1)
     splits = decode_splits(len(decode), nkv * (-(-g // 16)), max_kv_decode) if decode else 1

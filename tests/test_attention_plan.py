@@ -1,7 +1,8 @@
 """The host-side plan of the prefill attention kernel: which rows go to which block."""
 import random
 
-from jax_vllm_amd.parts.attention_backend import KEY_TILE, decode_splits, prefill_item_shape, prefill_work_items
+from jax_vllm_amd.parts.attention_backend import (KEY_TILE, decode_splits, pair_up_resident_items, prefill_item_shape,
+                                                   prefill_work_items)
 
 
 def _tiles(cl, m0, ql, g, rows, window):
@@ -46,6 +47,23 @@ def test_window_pairs_neighbours():
     assert sorted((a, b) for _, a, b in items) == [(m0, m0 + 64) for m0 in range(0, 512, 128)]
     items = prefill_work_items([512], [0], 1, 0, 64, 2, balance=False)
     assert [(a, b) for _, a, b in items] == [(m0, m0 + 64) for m0 in range(384, -1, -128)]   # heaviest first
+
+
+def test_items_that_are_all_on_the_chip_at_once_meet_heavy_with_light():
+    """Two blocks to a compute unit, handed out in the order of their numbers: item i and item i + n/2 share a
+    unit, so the lighter half runs in ascending order and every unit gets the same load."""
+    ql, g = 2048, 4
+    items = prefill_work_items([ql], [0], g, 0, 64, 2, balance=False)        # neighbours paired: loads 64, 62, ..., 2 tiles
+    loads = lambda its: [sum(_tiles(0, m0, ql, g, 64, 0) for m0 in (a, b) if m0 >= 0) for _, a, b in its]
+    paired = pair_up_resident_items(items, 256 // 8)                         # 512 blocks on 256 units: 32 items a round
+    assert sorted(paired) == sorted(items)
+    n = len(items)
+    sums = [x + y for x, y in zip(loads(paired)[:n // 2], loads(paired)[n // 2:])]
+    assert max(sums) - min(sums) <= 1
+    before = [x + y for x, y in zip(loads(items)[:n // 2], loads(items)[n // 2:])]
+    assert max(before) - min(before) >= 30
+    # 48 items of 8 blocks on 256 units: the 16 of the second round meet the 16 heaviest, lightest with heaviest
+    assert pair_up_resident_items(items[:48], 32) == items[:32] + items[32:48][::-1]
 
 
 def test_decode_splits_fill_the_chip_but_keep_a_tile_per_wave():
