@@ -60,7 +60,8 @@ def measure_decode(llm, batch, steps, warmup, rng, vocab, prompt_len=PROMPT_LEN)
     from jax_vllm_amd import SamplingParams
 
     prompts = [rng.integers(0, vocab, size=prompt_len).tolist() for _ in range(batch)]
-    sp = SamplingParams(max_new_tokens=warmup + steps + 128)
+    # the first requests decode while the others' prompts run, about two prompts a step: nobody may finish meanwhile
+    sp = SamplingParams(max_new_tokens=warmup + steps + max(128, batch))
     for p in prompts:
         llm.add_request(p, sp)
     while any(r.num_remaining > 1 or not r.output_ids for r in llm.scheduler.running) or llm.scheduler.waiting:
@@ -261,6 +262,8 @@ def main():
                     help="run only the first layers of the shape's (both numbers are reported in config)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--skip-points", action="store_true", help="measure the headline batch only")
+    ap.add_argument("--tune-library", action="store_true",
+                    help="prewarm the engine with the matrix library timing its own kernels (steps of more than 64 rows)")
     ap.add_argument("--no-kernel-share", action="store_true", help="leave out the per-kernel time shares")
     ap.add_argument("--only", choices=["prefill", "decode", "mixed", "long-prompt", "ttft", "calibrate"], default=None,
                     help="run one phase alone and print its result (for profiling); mixed: 32 running decodes "
@@ -314,7 +317,10 @@ def main():
     llm = LLM(cfg, random_seed=0, dtype=args.dtype, block_size=block, max_num_seqs=max_batch,
               max_model_len=max(MAX_CONTEXT, args.prompt_len + 2 * 1024),
               num_blocks=1 + max_batch * (-(-(args.prompt_len + 2 * 1024) // block)),
-              max_num_batched_tokens=max(PREFILL_TOKENS, max_batch), enable_prefix_cache=False)
+              max_num_batched_tokens=max(PREFILL_TOKENS, max_batch), enable_prefix_cache=False,
+              tune_library=args.tune_library)
+    if args.tune_library:
+        llm.prewarm()
     itemsize = 2 if args.dtype == "bf16" else 4
     wbytes, per_layer_params = weight_bytes(cfg, layers, itemsize)
     kv_per_token = llm.core.kv_bytes_per_token

@@ -37,6 +37,8 @@ class EngineConfig:
     enable_prefix_cache: bool = True     # reuse full pages of equal prompt prefixes
     use_hip_graphs: bool = True          # replay captured decode-only steps
     decode_ahead: bool = True            # start the decode step after a captured one before its tokens reach the host
+    tune_library: bool = False           # at prewarm, let the matrix library time its own kernels for the products it is given
+                                         # (steps of more than 64 rows) instead of taking its first guess
     seed: int = 0                        # default sampling seed
 
     def __post_init__(self):

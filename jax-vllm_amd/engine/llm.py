@@ -266,6 +266,21 @@ class LLM(Engine):
         t0 = time.perf_counter()
         from .core import _batch_bucket
 
+        tuning = self.config.tune_library and self.config.dtype == "bfloat16"
+        if tuning:
+            # The library's first guess is far off for 65..256 rows (8B sizes, 128 rows: down 66 us, timed choice 45;
+            # qkv at 256 rows 40 against 28).  Its timing pass runs at the first (eager) call of a shape, here and
+            # only here; it is switched off again below, so a shape first seen while serving takes the first guess.
+            # Buffers take turns while it times (512 MB), or it would time weights that sit in the cache.
+            import os
+            import tempfile
+
+            tunable = torch.cuda.tunable
+            tunable.set_filename(os.path.join(tempfile.gettempdir(), f"jax_vllm_amd_tuned_{os.getuid()}.csv"))
+            tunable.set_rotating_buffer_size(512)
+            tunable.enable(True)
+            tunable.tuning_enable(True)
+
         saved = (self.stats, self._next_id, self.core.cache.prefix_cache)
         self.core.cache.prefix_cache = False     # the warm-up prompts must not enter the prefix index
         self.stats = self.scheduler.stats = EngineStats()
@@ -279,6 +294,8 @@ class LLM(Engine):
                 first = False
                 self.generate([[0] * n] + [[0]] * (b - 1), SamplingParams(max_new_tokens=4))
         finally:
+            if tuning:
+                torch.cuda.tunable.tuning_enable(False)      # the choices made stay in use
             self.core.cache.prefix_cache = saved[2]
             self.stats, self._next_id = saved[0], saved[1]
             self.scheduler.stats = self.stats

@@ -1356,3 +1356,25 @@ def test_decode_steps_started_ahead_with_a_window_group_and_with_state(folders, 
         assert [len(o) for i, o in enumerate(outs[ahead]) if i != 2] == [70, 64, 30, 25]
         for i, (p, o) in enumerate(zip(prompts, outs[ahead])):
             _tokens_follow(dtype, plain, p, o, what=f"request {i} (ahead={ahead})")
+
+
+def test_prewarm_with_the_library_timing_its_own_kernels(folders):
+    """``tune_library``: during ``prewarm`` (and only then) the matrix library times its own kernels for the
+    products it is given.  Afterwards its timing pass is off again, and the tokens are the plain ones."""
+    from jax_vllm_amd import LLM, SamplingParams
+
+    cfg, w = plain_of(folders["B"])
+    rng = np.random.default_rng(31)
+    prompts = [rng.integers(0, cfg["vocab_size"], size=n).tolist() for n in (40, 23, 31)]
+    was = (torch.cuda.tunable.is_enabled(), torch.cuda.tunable.tuning_is_enabled())
+    try:
+        llm = LLM(folders["B"], dtype="bfloat16", block_size=16, max_num_seqs=24, max_model_len=128,
+                  max_num_batched_tokens=64, tune_library=True)
+        assert llm.prewarm() > 0
+        assert torch.cuda.tunable.is_enabled() and not torch.cuda.tunable.tuning_is_enabled()
+        got = llm.generate(prompts, SamplingParams(max_new_tokens=12))
+        for p, g in zip(prompts, got):
+            check_tokens_follow("bfloat16", cfg, w, p, g)
+    finally:
+        torch.cuda.tunable.tuning_enable(was[1])
+        torch.cuda.tunable.enable(was[0])
