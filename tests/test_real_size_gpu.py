@@ -332,3 +332,86 @@ def test_long_contexts_with_the_real_head_geometry(dtype, length):
     check_logits(dtype, np.concatenate(got), want, what=f"{length} tokens")
     core.finish_request("a")
     core.cache.check_invariants()
+
+
+# ------------------------------------------------------------------ one far token decides the logits
+NEEDLE_CONFIG = dict(CONFIG, num_hidden_layers=1, hidden_size=256, num_attention_heads=4, num_key_value_heads=2,
+                     intermediate_size=384, vocab_size=96)
+
+
+def needle_model():
+    """A one-layer model with heads of 128 whose weights are made so that ONE far token decides the last token's
+    logits: token NEEDLE's key and token ASK's query are both concentrated on the head element that the rotation
+    turns slowest, their q/k-norm weight there is 1.5, so ASK's score with NEEDLE is 11.3 * 1.5^2 = 25 while its
+    scores with the thousands of other keys stay below 8: ASK's attention output is NEEDLE's value, whatever else
+    the context holds.  Among random weights alone a lost page would move nothing that a bfloat16 bound sees."""
+    sized = Sized(NEEDLE_CONFIG, seed=9)
+    d, hid = 128, 256
+    slow = d // 2 - 1                                        # pairs with element d - 1; angle 1e6^(-126/128) a position
+    g = torch.Generator().manual_seed(3)
+    w = {n: t.clone() for n, t in sized.plain_w.items()}
+    p = "model.layers.0."
+    needle, ask = 90, 91
+    emb = 0.3 * torch.randn(96, hid, generator=g)
+    emb[:, :2] = 0.0
+    emb[needle] = 0.05 * torch.randn(hid, generator=g)
+    emb[needle, 0] = 4.0
+    emb[ask] = 0.05 * torch.randn(hid, generator=g)
+    emb[ask, 1] = 4.0
+    w["model.embed_tokens.weight"] = emb.cuda()
+    w[p + "input_layernorm.weight"] = torch.ones(hid).cuda()
+    for name, col, heads in (("k_proj", 0, 2), ("q_proj", 1, 4)):
+        m = 0.05 * torch.randn(heads * d, hid, generator=g)
+        m[:, :2] = 0.0
+        for h in range(heads):
+            m[h * d + slow, col] = 1.0
+        w[p + f"self_attn.{name}.weight"] = m.cuda()
+    for name in ("q_norm", "k_norm"):
+        v = torch.ones(d)
+        v[slow] = 1.5
+        w[p + f"self_attn.{name}.weight"] = v.cuda()
+    w[p + "self_attn.v_proj.weight"] = (0.3 * torch.randn(2 * d, hid, generator=g)).cuda()
+    w[p + "self_attn.o_proj.weight"] = (0.3 * torch.randn(hid, 4 * d, generator=g)).cuda()
+    w["lm_head.weight"] = (0.3 * torch.randn(96, hid, generator=g)).cuda()
+    sized.dev = {n: t.to(torch.bfloat16) for n, t in w.items()}
+    sized.plain_w = {n: t.float() for n, t in sized.dev.items()}
+    return sized, needle, ask
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("context,place", [(3000, 0), (3000, 1535), (3000, 1536), (3000, 2990), (700, 351), (5000, 4097)])
+def test_one_far_token_decides_the_logits(dtype, context, place):
+    """The prompt holds NEEDLE once, at ``place``; ASK comes as the last token of the last prompt portion, then as a
+    decoded token (a replayed step whose keys are shared out to several blocks), then once more after two other
+    tokens.  The oracle says that each of these rows depends on the needle (without it the logits move by more than a
+    quarter of their size), so an engine that loses, misplaces or misweights that one key among thousands is far
+    outside the bound of either precision."""
+    from jax_vllm_amd.engine.entries import StepEntry
+
+    sized, needle, ask = needle_model()
+    rng = np.random.default_rng(context + place)
+    toks = rng.integers(0, 90, size=context).tolist()
+    toks[place] = needle
+    toks += [ask, ask, 5, 17, ask]
+    rows = [context, context + 1, context + 4]
+    want = sized.plain(toks, rows)
+    without = list(toks)
+    without[place] = 7
+    moved = np.abs(sized.plain(without, rows) - want).max(axis=1)
+    scale = float(np.abs(want).max())
+    assert (moved > 0.25 * scale).all(), f"the oracle's rows do not depend on the needle enough: {moved} of {scale}"
+    core = make_core(None, dtype, 16, pages=-(-len(toks) // 16) + 2, seqs=2, model=sized.model(dtype), graphs=True)
+    core.start_request("a")
+    got = []
+    for at in range(0, context + 1, 1024):
+        part = toks[at:min(at + 1024, context + 1)]
+        last = at + len(part) == context + 1
+        out = core.run([StepEntry("a", part, [len(part) - 1] if last else [])])
+        if last:
+            got.append(out.cpu().numpy())
+    for i in range(context + 1, len(toks)):
+        out = core.run([StepEntry("a", toks[i:i + 1], [0])]).cpu().numpy()
+        if i in rows:
+            got.append(out)
+    assert core.graph_replays >= 2
+    check_logits(dtype, np.concatenate(got), want, scale, f"needle at {place} of {context}")
