@@ -16,9 +16,27 @@ __global__ void embedding_kernel(float* __restrict__ h, const T* __restrict__ ta
   const T* row = table + (long long)(inside ? id : 0) * hidden;
   float* out = h + t * hidden;
   const float nan = __builtin_nanf("");
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
-    const float v = to_f32(row[i]);
-    out[i] = inside ? v : nan;
+  // 16 bytes of the table a lane where the row allows it (a width that is a multiple of the pieces'
+  // elements keeps every row of table and of h aligned), element by element otherwise
+  constexpr int V = 16 / sizeof(T);
+  if (hidden % V == 0) {
+    typedef T tv __attribute__((ext_vector_type(V)));
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    for (int i = threadIdx.x * V; i < hidden; i += blockDim.x * V) {
+      const tv v = *(const tv*)(row + i);
+#pragma unroll
+      for (int j = 0; j < V; j += 4) {
+        f4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = inside ? to_f32(v[j + e]) : nan;
+        *(f4*)(out + i + j) = o;
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+      const float v = to_f32(row[i]);
+      out[i] = inside ? v : nan;
+    }
   }
 }
 

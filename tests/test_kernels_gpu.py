@@ -27,7 +27,7 @@ def randn(*shape, dtype=torch.float32, seed=0, scale=1.0):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hidden,vocab", [(72, 333), (4096, 1000)])
+@pytest.mark.parametrize("hidden,vocab", [(72, 333), (4096, 1000), (70, 50), (12, 19)])
 def test_embedding(dtype, hidden, vocab):
     table = randn(vocab, hidden, dtype=dtype)
     ids = torch.tensor([0, vocab - 1, 5, 5, 17], dtype=torch.int32).cuda()
