@@ -698,14 +698,15 @@ def test_attention_edges_of_visibility(edge, kernel):
 
 
 @pytest.mark.parametrize("kernel", ["prefill", "decode1", "decode4", "decode16"])
+@pytest.mark.parametrize("heads", [(8, 2), (16, 2)], ids=["4-a-group", "8-a-group"])
 @pytest.mark.parametrize("ctx", [8191, 16400, 32767])
-def test_mfma_attention_over_long_contexts_at_head_size_128(kernel, ctx):
-    """Heads of 128, 4 per kv head, pages of 16, behind 8 k to 32 k keys.  Among thousands of random
+def test_mfma_attention_over_long_contexts_at_head_size_128(kernel, ctx, heads):
+    """Heads of 128, 4 or 8 per kv head (the 8B/14B and the 32B geometry), pages of 16, behind 8 k to 32 k keys.  Among thousands of random
     keys a missing page would change nothing that a tolerance sees, so every checked query has TWO
     loud keys far apart (the first key, a page's last slot in the middle, a page's first slot, the
     newest key): its output is the mean of their two values, and a key that is lost, read from a
     wrong page or merged with a wrong weight shows as an error of half a value."""
-    nq, nkv, d, page_size = 8, 2, 128, 16
+    (nq, nkv), d, page_size = heads, 128, 16
     scale = 1.0 / math.sqrt(d)
     bf = torch.bfloat16
     decode = kernel.startswith("decode")

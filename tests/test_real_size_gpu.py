@@ -10,7 +10,10 @@ Then the shapes that the measurement program times, again against the plain impl
 decode-only steps of 8, 24 and 64 requests behind prompts of about 1,024 tokens, recorded and
 replayed and started ahead of their tokens; one prompt of 2,048 tokens whole, cut, and behind a
 prefix taken from the cache; contexts of 8,300 and 20,000 tokens on a narrow model with the real
-head geometry.  The plain implementation runs on the GPU here, in torch's exact float32."""
+head geometry; one far token that decides the logits; and the workloads of the larger
+configurations: running decodes joined by long prompts in portions with a shared prefix (14B
+sizes), decodes behind 16,400 tokens (32B sizes).  The plain implementation runs on the GPU here,
+in torch's exact float32."""
 import numpy as np
 import pytest
 import torch
@@ -415,3 +418,83 @@ def test_one_far_token_decides_the_logits(dtype, context, place):
             got.append(out)
     assert core.graph_replays >= 2
     check_logits(dtype, np.concatenate(got), want, scale, f"needle at {place} of {context}")
+
+
+# ------------------------------------------------------------------ the workloads of the larger configurations
+def _follows(sized, prompt, out, dtype, what):
+    """Every generated token is the plain implementation's choice given all before it (bfloat16: within 4 % of the
+    largest logit of the maximum)."""
+    rows = list(range(len(prompt) - 1, len(prompt) + len(out) - 1))
+    logits = sized.plain(prompt + out[:-1], rows)
+    for k, t in enumerate(out):
+        margin = float(logits[k].max() - logits[k][t])
+        allowed = (1e-4 if dtype == "float32" else 0.04) * float(np.abs(logits[k]).max())
+        assert margin <= allowed, f"{what}, token {k}: engine's {t} is {margin} below the plain maximum"
+
+
+@pytest.mark.parametrize("dtype,running,longest", [("bfloat16", 32, 4096), ("float32", 8, 1500)])
+def test_running_decodes_joined_by_long_prompts_in_portions_with_a_shared_prefix(dtype, running, longest):
+    """The continuous-batching mix of the 14B sizes (two layers): requests decoding at contexts drawn from
+    [512, longest] are joined by 4 prompts (3,000 tokens, or 1,200 in 32-bit), prefilled in portions of 512 under a
+    budget of 2,048 tokens a step beside the decodes; two of the prompts share their first 1,024 tokens, which the
+    second one must find in the cache.  Every token of every request against the plain implementation."""
+    from jax_vllm_amd.engine.llm import LLM
+    from jax_vllm_amd.engine.request import SamplingParams
+
+    sized = Sized(CONFIG_14B, seed=2)
+    vocab = sized.cfg.vocab_size
+    rng = np.random.default_rng(running)
+    join_len = 3000 if dtype == "bfloat16" else 1200
+    llm = LLM(sized.model(dtype), dtype=dtype, block_size=16, max_num_seqs=running + 4, max_model_len=longest + 128,
+              num_blocks=1 + running * (-(-(longest + 64) // 16)) + 4 * (-(-(join_len + 64) // 16)),
+              max_num_batched_tokens=2048, max_chunk=512, enable_prefix_cache=True)
+    first = [rng.integers(0, vocab, size=int(n)).tolist() for n in rng.integers(512, longest + 1, size=running)]
+    rids = [llm.add_request(p, SamplingParams(max_new_tokens=40)) for p in first]
+    outs = {}
+
+    def step():
+        for e in llm.step():
+            outs.setdefault(e.request_id, []).append(e.token)
+
+    while any(not outs.get(r) for r in rids):
+        step()
+    for _ in range(4):                       # decode steps of the running requests alone
+        step()
+    prefix = rng.integers(0, vocab, size=1024).tolist()
+    joining = [rng.integers(0, vocab, size=join_len).tolist() for _ in range(4)]
+    for p in joining[-2:]:
+        p[:1024] = prefix
+    hits = llm.stats.cache_hit_tokens
+    new = [llm.add_request(p, SamplingParams(max_new_tokens=6)) for p in joining]
+    mixed_steps = 0
+    while llm.has_work():
+        before = llm.stats.prefill_tokens, llm.stats.decode_tokens
+        step()
+        mixed_steps += llm.stats.prefill_tokens > before[0] and llm.stats.decode_tokens > before[1]
+    assert llm.stats.cache_hit_tokens - hits == 1024 and mixed_steps >= 2
+    assert llm.stats.max_batched_tokens <= 2048 and llm.stats.graph_replays > 0 and llm.stats.preemptions == 0
+    llm.core.cache.check_invariants()
+    for i, (p, r) in enumerate(zip(first + joining, rids + new)):
+        assert len(outs[r]) == (40 if i < running else 6)
+        _follows(sized, p, outs[r], dtype, f"request {i}")
+
+
+def test_decodes_behind_16k_tokens_at_the_32b_head_geometry():
+    """The long-context workload of the 32B sizes (two layers, bfloat16): requests behind prompts of about 16,400
+    tokens decode together, their steps recorded and replayed (8 query heads share a kv head, block tables of more
+    than a thousand pages).  Every token against the plain implementation."""
+    from jax_vllm_amd.engine.llm import LLM
+    from jax_vllm_amd.engine.request import SamplingParams
+
+    sized = Sized(CONFIG_32B, seed=3)
+    vocab = sized.cfg.vocab_size
+    rng = np.random.default_rng(16)
+    lens = [16384, 16400, 16385, 16431]
+    prompts = [rng.integers(0, vocab, size=n).tolist() for n in lens]
+    llm = LLM(sized.model("bfloat16"), dtype="bfloat16", block_size=16, max_num_seqs=4, max_model_len=16512,
+              max_num_batched_tokens=2048, enable_prefix_cache=False)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=10))
+    assert llm.stats.graph_replays >= 6 and llm.stats.steps_ahead >= 6
+    for i, (p, o) in enumerate(zip(prompts, outs)):
+        assert len(o) == 10
+        _follows(sized, p, o, "bfloat16", f"request {i}")
